@@ -1,0 +1,207 @@
+/*
+ * llmi_hip.h -- C ABI of the gfx950 (MI355X) decode-attention backend.
+ *
+ * Plain pointers and sizes only. Every entry point returns LLMI_OK (0) or a
+ * negative llmi_status; nothing here aborts the process. All device work is
+ * enqueued on the caller's stream and borrows the caller's buffers until that
+ * stream has been synchronised. Not thread-safe per pool / per stream, like
+ * the engine it plugs into (one host thread, one stream).
+ *
+ * Reference interfaces replaced (paths relative to the reference checkout):
+ *   llmi_hip_mha_decode           kernel::mha_kernel_cu
+ *                                 code/source/op/kernel/cuda/mha_kernel.cu:440-529
+ *                                 (registry slot kernel_interface.h:168-183,
+ *                                 kernel_interface.cpp:181-190; caller
+ *                                 code/source/op/mha.cpp:54-56)
+ *   llmi_hip_mha_workspace_bytes  the KVSplitOutput buffer sizing
+ *                                 code/source/model/qwen3_fused.cpp:502-503
+ *   llmi_hip_mha_plan             the dispatch arithmetic inside mha_kernel_cu
+ *                                 mha_kernel.cu:505-517
+ *   llmi_hip_qk_norm_rope_append  kernel::fused_qk_norm_rope_kernel_cu
+ *                                 code/source/op/kernel/cuda/rmsnorm_kernel.cu:248-290
+ *                                 plus the K/V row placement of
+ *                                 Model::slice_kv_cache code/source/model/model.cpp:90-107
+ *   llmi_hip_sincos_table         kernel::sin_cos_cache_precompute_cu
+ *                                 code/source/op/kernel/cuda/rope_kernel.cu:23-46
+ *   llmi_hip_kv_restride          (new) converts a position-major cache
+ *                                 (qwen3_fused.cpp:488-491) to the head-major layout
+ *   llmi_pool_* / llmi_hip_pool_* base::CUDADeviceAllocator::allocate / release
+ *                                 code/source/base/alloc_cu.cpp:7-119
+ *   llmi_hip_memcpy / memset_zero base::DeviceAllocator::memcpy / memset_zero
+ *                                 code/source/base/alloc.cpp:11-72
+ */
+#ifndef LLMI_HIP_H
+#define LLMI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLMI_HIP_ABI_VERSION 1
+
+typedef enum llmi_status {
+    LLMI_OK = 0,
+    LLMI_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                       */
+    LLMI_ERR_HEAD_DIM = -2,       /* head_dim != 128 (mha_kernel.cu:478-479)          */
+    LLMI_ERR_KV_DIM = -3,         /* kv_dim not a positive multiple of head_dim / 8   */
+    LLMI_ERR_ALIGNMENT = -4,      /* q/K/V/out not 16-byte aligned (mha_kernel.cu:495-498) */
+    LLMI_ERR_POS_RANGE = -5,      /* pos < 0 or pos >= max_seq_len (mha_kernel.cu:473-474) */
+    LLMI_ERR_WORKSPACE = -6,      /* workspace missing or too small for the split path */
+    LLMI_ERR_HEAD_GROUP = -7,     /* head_num != kv_mul * (kv_dim/head_dim), or kv_mul > 16 */
+    LLMI_ERR_LAYOUT = -8,         /* unknown kv_layout                                 */
+    LLMI_ERR_INVALID_ARG = -9,    /* any other out-of-range scalar                     */
+    LLMI_ERR_LAUNCH = -10,        /* hipGetLastError() after a launch / a HIP call failed */
+    LLMI_ERR_UNKNOWN_POINTER = -11, /* pool free of a pointer the pool does not own    */
+    LLMI_ERR_OUT_OF_MEMORY = -12  /* backing allocator failed                          */
+} llmi_status;
+
+/* KV-cache layouts. Both hold bf16 bit patterns (uint16_t) and head_dim = 128. */
+enum {
+    /* the reference's: [layer][max_seq_len][kv_head][128]  (qwen3_fused.cpp:488-491) */
+    LLMI_KV_LAYOUT_POS_MAJOR = 0,
+    /* re-strided:      [layer][kv_head][max_seq_len][128] -- each KV head's rows are contiguous */
+    LLMI_KV_LAYOUT_HEAD_MAJOR = 1
+};
+
+enum { LLMI_PATH_AUTO = 0, LLMI_PATH_SINGLE_PASS = 1, LLMI_PATH_SPLIT = 2 };
+
+typedef struct llmi_mha_args {
+    const void* query;        /* device, bf16 [head_num*head_dim]                        */
+    const void* key_cache;    /* device, bf16, base of the whole cache (all layers)      */
+    const void* value_cache;  /* device, bf16                                            */
+    void* workspace;          /* device, fp32 split partials; may be NULL if single-pass */
+    size_t workspace_bytes;   /* size of workspace                                       */
+    void* output;             /* device, bf16 [head_num*head_dim]                        */
+    float* output_f32;        /* optional device fp32 [head_num*head_dim] tap of the
+                                 result before bf16 rounding; NULL in production         */
+    int32_t layer_id;
+    int32_t pos;              /* attends to positions 0..pos                             */
+    int32_t kv_dim;           /* kv_heads * head_dim                                     */
+    int32_t kv_mul;           /* query heads per KV head                                 */
+    int32_t head_num;         /* query heads                                             */
+    int32_t head_dim;         /* must be 128                                             */
+    int32_t max_seq_len;      /* positions per layer in the cache                        */
+    int32_t kv_layout;        /* LLMI_KV_LAYOUT_*                                        */
+    int32_t force_path;       /* LLMI_PATH_*; AUTO picks by context length               */
+    int32_t num_splits;       /* 0 = auto; otherwise the KV split count of the split path */
+    int32_t waves_per_group;  /* 0 = auto; 1,2,4,8 wavefronts per workgroup (tuning)     */
+    void* stream;             /* hipStream_t, NULL = the null stream                     */
+} llmi_mha_args;
+
+typedef struct llmi_mha_plan {
+    int32_t path;             /* LLMI_PATH_SINGLE_PASS or LLMI_PATH_SPLIT                */
+    int32_t num_splits;       /* 1 for single-pass                                       */
+    int32_t rows_per_split;   /* multiple of 16                                          */
+    int32_t waves_per_group;
+    int32_t group_pad;        /* query heads per KV head rounded up to 1,2,4,8,16        */
+    size_t workspace_needed;  /* bytes of workspace this plan uses (0 for single-pass)   */
+} llmi_mha_plan;
+
+/* Validates args and reports what llmi_hip_mha_decode would launch. Makes no
+ * HIP call, so it also works on a host without a GPU. */
+int llmi_hip_mha_plan(const llmi_mha_args* args, llmi_mha_plan* plan);
+
+/* Decode attention for one layer and one new token: for every query head h,
+ * out[h] = softmax(q[h].K[h/kv_mul]^T / sqrt(128)) . V[h/kv_mul] over positions
+ * 0..pos, bf16 in, fp32 accumulate, bf16 out. Enqueues 1 kernel (single-pass)
+ * or 2 (split + combine). Allocates nothing; safe under stream capture. */
+int llmi_hip_mha_decode(const llmi_mha_args* args);
+
+/* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */
+size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len);
+
+typedef struct llmi_qk_norm_rope_args {
+    void* query;              /* device bf16 [head_num*128], normalised+rotated in place  */
+    const void* key_new;      /* device bf16 [kv_dim]: this token's K row (pre-norm)      */
+    const void* value_new;    /* device bf16 [kv_dim]: this token's V row, or NULL if the
+                                 V row is already in the cache                            */
+    void* key_cache;          /* device bf16 cache base; row (layer_id,pos) is written    */
+    void* value_cache;        /* device bf16 cache base; written when value_new != NULL   */
+    const void* norm_weight;  /* device bf16 [2*128]: q_norm then k_norm                  */
+    const float* sin_cache;   /* device fp32 [max_seq_len][64]                            */
+    const float* cos_cache;   /* device fp32 [max_seq_len][64]                            */
+    int32_t layer_id;
+    int32_t pos;
+    int32_t kv_dim;
+    int32_t head_num;
+    int32_t head_dim;         /* must be 128 */
+    int32_t max_seq_len;
+    int32_t kv_layout;
+    float eps;                /* 1e-6 in the reference (rmsnorm_kernel.cu:284)            */
+    void* stream;
+} llmi_qk_norm_rope_args;
+
+/* Per-head RMSNorm * weight then half-rotation RoPE on the query (in place)
+ * and on this token's K row, which is written to its cache slot for
+ * (layer_id, pos) in the given layout, together with the V row. When key_new
+ * points at the cache slot itself the K row is transformed in place, which is
+ * what the reference does. One kernel, no allocation. */
+int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* args);
+
+/* sin/cos(pos * 1e6^(-2i/head_dim)) for pos < max_seq_len, i < head_dim/2. */
+int llmi_hip_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim,
+                          int32_t max_seq_len, void* stream);
+
+/* Copies rows 0..num_pos-1 of every layer from a position-major cache into a
+ * head-major one (src and dst must not overlap). */
+int llmi_hip_kv_restride(const void* src_pos_major, void* dst_head_major, int32_t layer_num,
+                         int32_t max_seq_len, int32_t kv_dim, int32_t head_dim, int32_t num_pos,
+                         void* stream);
+
+/* ---- pooled device allocator ------------------------------------------- */
+
+typedef struct llmi_pool llmi_pool;
+/* Backing allocator: returns 0 and sets *ptr on success. */
+typedef int (*llmi_backing_alloc_fn)(void** ptr, size_t bytes, void* user);
+typedef int (*llmi_backing_free_fn)(void* ptr, void* user);
+
+typedef struct llmi_pool_stats {
+    size_t backing_allocs;    /* calls that reached the backing allocator          */
+    size_t reuses;            /* allocations served from a free block              */
+    size_t big_busy_blocks, big_free_blocks;
+    size_t small_busy_blocks, small_free_blocks;
+    size_t big_busy_bytes, big_free_bytes;
+    size_t small_busy_bytes, small_free_bytes;
+} llmi_pool_stats;
+
+/* A pool with the reference's policy (alloc_cu.cpp:7-119): requests above
+ * 1 MiB reuse the smallest free big block that fits with less than 1 MiB of
+ * slack; requests of 1 MiB or less reuse the smallest free small block that
+ * fits; released blocks go back to the free sets and are never returned to
+ * the backing allocator until llmi_pool_trim / llmi_pool_destroy. */
+llmi_pool* llmi_pool_create(llmi_backing_alloc_fn alloc_fn, llmi_backing_free_fn free_fn,
+                            void* user);
+void llmi_pool_destroy(llmi_pool* pool);
+/* NULL for bytes == 0 or when the backing allocator fails. */
+void* llmi_pool_alloc(llmi_pool* pool, size_t bytes);
+/* LLMI_OK (also for NULL), LLMI_ERR_UNKNOWN_POINTER for a pointer that is not busy in the pool. */
+int llmi_pool_free(llmi_pool* pool, void* ptr);
+/* Hands every free block back to the backing allocator; returns bytes released. */
+size_t llmi_pool_trim(llmi_pool* pool);
+int llmi_pool_get_stats(const llmi_pool* pool, llmi_pool_stats* stats);
+
+/* The process-wide pool over hipMalloc/hipFree on the current device. */
+llmi_pool* llmi_hip_default_pool(void);
+void* llmi_hip_pool_alloc(size_t bytes);
+int llmi_hip_pool_free(void* ptr);
+
+/* kind: 0 host->host, 1 host->device, 2 device->host, 3 device->device
+ * (base::MemcpyKind, code/include/base/alloc.h:10-15). A NULL stream copies
+ * synchronously; need_sync adds a device synchronise. */
+int llmi_hip_memcpy(void* dst, const void* src, size_t bytes, int32_t kind, void* stream,
+                    int32_t need_sync);
+int llmi_hip_memset_zero(void* ptr, size_t bytes, void* stream, int32_t need_sync);
+
+/* ---- misc ---------------------------------------------------------------- */
+int llmi_hip_abi_version(void);
+const char* llmi_hip_strerror(int status);
+/* The last HIP error string seen by this library on the calling thread ("" if none). */
+const char* llmi_hip_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMI_HIP_H */

@@ -1,0 +1,67 @@
+"""Builds libllmi_hip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(HERE, "libllmi_hip.so")
+HOST_LIB_PATH = os.path.join(HERE, "libllmi_host.so")
+
+HIP_SOURCES = ["mha_decode.hip", "qk_norm_rope.hip", "c_api.cpp", "pool.cpp"]
+
+# -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("build failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_hip_library(verbose=False):
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES] + ["-o", LIB_PATH]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+def build_host_library(verbose=False):
+    """The C++17 mirror of the reference's tensor/op/registry interface, linked against libllmi_hip.so."""
+    host_dir = os.path.join(CSRC, "host")
+    if not os.path.isdir(host_dir):
+        return None
+    srcs = sorted(os.path.join(host_dir, f) for f in os.listdir(host_dir) if f.endswith(".cpp"))
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    cmd = [hipcc, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-command-line-argument",
+           "-I" + os.path.join(ROOT, "include"), "-I" + host_dir] + srcs
+    cmd += ["-L" + HERE, "-lllmi_hip", "-Wl,-rpath,$ORIGIN", "-o", HOST_LIB_PATH]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return HOST_LIB_PATH
+
+
+def build_all(verbose=False):
+    paths = [build_hip_library(verbose)]
+    host = build_host_library(verbose)
+    if host:
+        paths.append(host)
+    return paths
+
+
+if __name__ == "__main__":
+    for p in build_all(verbose=True):
+        print("built", p)
+    sys.exit(0)

@@ -1,0 +1,296 @@
+// C ABI of libllmi_hip.so: argument validation, the context-length dispatch,
+// the hipMalloc-backed default pool and the copy helpers. The kernels live in
+// mha_decode.hip and qk_norm_rope.hip.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "llmi_hip.h"
+#include "llmi_internal.h"
+#include "pool.h"
+
+namespace llmi {
+
+namespace {
+thread_local std::string g_last_error;
+
+// Context lengths up to this run as one workgroup per KV head; longer ones are
+// split over the 256 CUs. (The reference's threshold is 128 with 32-position
+// splits, mha_kernel.cu:507-517; here a split costs a second launch and a
+// workspace round trip, and one workgroup already streams a whole KV head.)
+constexpr int kSinglePassMaxLen = 256;
+// Workgroups the split path aims for: a few per CU so every CU has loads in flight.
+constexpr int kTargetGroups = 1024;
+constexpr int kTile = 16;
+
+inline int pow2_ceil(int x) {
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+inline int pow2_floor(int x) {
+    int p = 1;
+    while (p * 2 <= x) p <<= 1;
+    return p;
+}
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+}  // namespace
+
+int record_hip_error(hipError_t err, const char* what) {
+    if (err == hipSuccess) return LLMI_OK;
+    g_last_error = std::string(what) + ": " + hipGetErrorString(err);
+    return LLMI_ERR_LAUNCH;
+}
+
+int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
+
+static int validate_mha(const llmi_mha_args* a) {
+    if (!a) return LLMI_ERR_NULL_POINTER;
+    if (!a->query || !a->key_cache || !a->value_cache || !a->output) return LLMI_ERR_NULL_POINTER;
+    if (a->head_dim != 128) return LLMI_ERR_HEAD_DIM;                               // mha_kernel.cu:478-479
+    if (a->kv_dim <= 0 || a->kv_dim % a->head_dim != 0) return LLMI_ERR_KV_DIM;     // mha_kernel.cu:494
+    if (a->kv_mul < 1 || a->kv_mul > kMaxGroup) return LLMI_ERR_HEAD_GROUP;
+    if (a->head_num != a->kv_mul * (a->kv_dim / a->head_dim)) return LLMI_ERR_HEAD_GROUP;
+    if (a->max_seq_len <= 0 || a->layer_id < 0) return LLMI_ERR_INVALID_ARG;
+    if (a->pos < 0 || a->pos >= a->max_seq_len) return LLMI_ERR_POS_RANGE;          // mha_kernel.cu:473-474
+    if (a->kv_layout != LLMI_KV_LAYOUT_POS_MAJOR && a->kv_layout != LLMI_KV_LAYOUT_HEAD_MAJOR)
+        return LLMI_ERR_LAYOUT;
+    if (!aligned16(a->query) || !aligned16(a->key_cache) || !aligned16(a->value_cache) || !aligned16(a->output))
+        return LLMI_ERR_ALIGNMENT;                                                  // mha_kernel.cu:495-498
+    if (a->workspace && !aligned16(a->workspace)) return LLMI_ERR_ALIGNMENT;
+    if (a->output_f32 && (reinterpret_cast<uintptr_t>(a->output_f32) & 3u)) return LLMI_ERR_ALIGNMENT;
+    if (a->force_path < LLMI_PATH_AUTO || a->force_path > LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
+    if (a->num_splits < 0 || a->num_splits > kMaxSplits) return LLMI_ERR_INVALID_ARG;
+    const int w = a->waves_per_group;
+    if (!(w == 0 || w == 1 || w == 2 || w == 4 || w == 8)) return LLMI_ERR_INVALID_ARG;
+    return LLMI_OK;
+}
+
+static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
+    if (int rc = validate_mha(a)) return rc;
+    const int seq_len = a->pos + 1;
+    const int tiles = ceil_div(seq_len, kTile);
+    const int n_kv = a->kv_dim / a->head_dim;
+    const int group_pad = pow2_ceil(a->kv_mul);
+    int max_waves = pow2_floor(kMaxGroupWaves / group_pad);
+    if (max_waves > kMaxWaves) max_waves = kMaxWaves;
+    if (a->waves_per_group > max_waves) return LLMI_ERR_INVALID_ARG;
+    const size_t per_split = (size_t)a->head_num * (a->head_dim + 2) * sizeof(float);
+
+    int path = a->force_path;
+    if (path == LLMI_PATH_AUTO) {
+        if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
+        else if (a->num_splits > 1) path = LLMI_PATH_SPLIT;
+        else path = seq_len <= kSinglePassMaxLen ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT;
+    }
+
+    int num_splits = 1, tiles_per_split = tiles, waves;
+    if (path == LLMI_PATH_SPLIT) {
+        waves = a->waves_per_group ? a->waves_per_group : (max_waves < 4 ? max_waves : 4);
+        int want = a->num_splits;
+        if (want == 0) {
+            // Auto: a few workgroups per CU, at least one tile per wave, and
+            // no more splits than the caller's workspace can hold.
+            want = kTargetGroups / n_kv;
+            if (want < 2) want = 2;
+            if (want > kMaxSplits) want = kMaxSplits;
+            const size_t cap = a->workspace ? a->workspace_bytes / per_split : 0;
+            if (cap < 2) return LLMI_ERR_WORKSPACE;
+            if ((size_t)want > cap) want = (int)cap;
+            tiles_per_split = ceil_div(tiles, want);
+            if (tiles_per_split < waves) tiles_per_split = waves;
+        } else {
+            tiles_per_split = ceil_div(tiles, want);
+        }
+        num_splits = ceil_div(tiles, tiles_per_split);  // no empty splits
+        if (num_splits > 1) {
+            if (!a->workspace || a->workspace_bytes < per_split * (size_t)num_splits) return LLMI_ERR_WORKSPACE;
+        }
+    }
+    if (num_splits == 1) {
+        path = LLMI_PATH_SINGLE_PASS;
+        tiles_per_split = tiles;
+        if (a->waves_per_group) {
+            waves = a->waves_per_group;
+        } else {
+            waves = pow2_ceil(tiles);
+            if (waves > kMaxWaves) waves = kMaxWaves;
+            if (waves > max_waves) waves = max_waves;
+        }
+    }
+
+    p->path = path;
+    p->num_splits = num_splits;
+    p->rows_per_split = tiles_per_split * kTile;
+    p->waves_per_group = waves;
+    p->group_pad = group_pad;
+    p->workspace_needed = num_splits > 1 ? per_split * (size_t)num_splits : 0;
+    return LLMI_OK;
+}
+
+}  // namespace llmi
+
+using namespace llmi;
+
+extern "C" {
+
+int llmi_hip_mha_plan(const llmi_mha_args* args, llmi_mha_plan* plan) {
+    if (!plan) return LLMI_ERR_NULL_POINTER;
+    return make_plan(args, plan);
+}
+
+int llmi_hip_mha_decode(const llmi_mha_args* args) {
+    llmi_mha_plan plan;
+    if (int rc = make_plan(args, &plan)) return rc;
+    return launch_mha_decode(*args, plan);
+}
+
+size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len) {
+    if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
+    int splits = (max_seq_len + kTile - 1) / kTile;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    return (size_t)head_num * (size_t)splits * (size_t)(head_dim + 2) * sizeof(float);
+}
+
+int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {
+    if (!a) return LLMI_ERR_NULL_POINTER;
+    if (!a->query || !a->key_new || !a->key_cache || !a->norm_weight || !a->sin_cache || !a->cos_cache)
+        return LLMI_ERR_NULL_POINTER;
+    if (a->value_new && !a->value_cache) return LLMI_ERR_NULL_POINTER;
+    if (a->head_dim != 128) return LLMI_ERR_HEAD_DIM;                                // rmsnorm_kernel.cu:274
+    if (a->kv_dim <= 0 || a->kv_dim % a->head_dim != 0) return LLMI_ERR_KV_DIM;
+    if (a->head_num <= 0 || a->max_seq_len <= 0 || a->layer_id < 0) return LLMI_ERR_INVALID_ARG;
+    if (a->pos < 0 || a->pos >= a->max_seq_len) return LLMI_ERR_POS_RANGE;
+    if (a->kv_layout != LLMI_KV_LAYOUT_POS_MAJOR && a->kv_layout != LLMI_KV_LAYOUT_HEAD_MAJOR)
+        return LLMI_ERR_LAYOUT;
+    const void* ptrs[] = {a->query, a->key_new, a->value_new, a->key_cache, a->value_cache, a->norm_weight};
+    for (const void* p : ptrs)
+        if (p && (reinterpret_cast<uintptr_t>(p) & 3u)) return LLMI_ERR_ALIGNMENT;
+    if (!(a->eps >= 0.0f)) return LLMI_ERR_INVALID_ARG;
+    return launch_qk_norm_rope_append(*a);
+}
+
+int llmi_hip_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,
+                          void* stream) {
+    if (!sin_cache || !cos_cache) return LLMI_ERR_NULL_POINTER;
+    if (head_dim <= 0 || head_dim % 2 != 0) return LLMI_ERR_HEAD_DIM;
+    if (max_seq_len <= 0) return LLMI_ERR_INVALID_ARG;
+    return launch_sincos_table(sin_cache, cos_cache, head_dim, max_seq_len, static_cast<hipStream_t>(stream));
+}
+
+int llmi_hip_kv_restride(const void* src, void* dst, int32_t layer_num, int32_t max_seq_len, int32_t kv_dim,
+                         int32_t head_dim, int32_t num_pos, void* stream) {
+    if (!src || !dst) return LLMI_ERR_NULL_POINTER;
+    if (head_dim != 128) return LLMI_ERR_HEAD_DIM;
+    if (kv_dim <= 0 || kv_dim % head_dim != 0) return LLMI_ERR_KV_DIM;
+    if (layer_num <= 0 || max_seq_len <= 0) return LLMI_ERR_INVALID_ARG;
+    if (num_pos < 0 || num_pos > max_seq_len) return LLMI_ERR_POS_RANGE;
+    if (!aligned16(src) || !aligned16(dst)) return LLMI_ERR_ALIGNMENT;
+    if (src == dst) return LLMI_ERR_INVALID_ARG;
+    return launch_kv_restride(src, dst, layer_num, max_seq_len, kv_dim, head_dim, num_pos,
+                              static_cast<hipStream_t>(stream));
+}
+
+/* ---- pool ---------------------------------------------------------------- */
+
+llmi_pool* llmi_pool_create(llmi_backing_alloc_fn alloc_fn, llmi_backing_free_fn free_fn, void* user) {
+    if (!alloc_fn || !free_fn) return nullptr;
+    return new (std::nothrow) llmi_pool(alloc_fn, free_fn, user);
+}
+
+void llmi_pool_destroy(llmi_pool* pool) { delete pool; }
+
+void* llmi_pool_alloc(llmi_pool* pool, size_t bytes) { return pool ? pool->allocate(bytes) : nullptr; }
+
+int llmi_pool_free(llmi_pool* pool, void* ptr) { return pool ? pool->release(ptr) : LLMI_ERR_NULL_POINTER; }
+
+size_t llmi_pool_trim(llmi_pool* pool) { return pool ? pool->trim() : 0; }
+
+int llmi_pool_get_stats(const llmi_pool* pool, llmi_pool_stats* stats) {
+    if (!pool || !stats) return LLMI_ERR_NULL_POINTER;
+    pool->stats(stats);
+    return LLMI_OK;
+}
+
+static int hip_backing_alloc(void** ptr, size_t bytes, void*) {
+    hipError_t err = hipMalloc(ptr, bytes);
+    if (err != hipSuccess) {
+        record_hip_error(err, "hipMalloc");
+        (void)hipGetLastError();
+        *ptr = nullptr;
+        return LLMI_ERR_OUT_OF_MEMORY;
+    }
+    return 0;
+}
+
+static int hip_backing_free(void* ptr, void*) { return record_hip_error(hipFree(ptr), "hipFree"); }
+
+llmi_pool* llmi_hip_default_pool(void) {
+    // Leaked on purpose: device memory is reclaimed by the driver at process
+    // exit, and freeing from a static destructor can run after HIP has shut down.
+    static llmi_pool* pool = new llmi_pool(hip_backing_alloc, hip_backing_free, nullptr);
+    return pool;
+}
+
+void* llmi_hip_pool_alloc(size_t bytes) { return llmi_hip_default_pool()->allocate(bytes); }
+
+int llmi_hip_pool_free(void* ptr) { return llmi_hip_default_pool()->release(ptr); }
+
+int llmi_hip_memcpy(void* dst, const void* src, size_t bytes, int32_t kind, void* stream, int32_t need_sync) {
+    if (!dst || !src) return LLMI_ERR_NULL_POINTER;  // alloc.cpp:12-13
+    if (bytes == 0) return LLMI_OK;                  // alloc.cpp:15-17
+    if (kind == 0) {
+        std::memcpy(dst, src, bytes);  // alloc.cpp:26-27
+        return LLMI_OK;
+    }
+    hipMemcpyKind k;
+    if (kind == 1) k = hipMemcpyHostToDevice;
+    else if (kind == 2) k = hipMemcpyDeviceToHost;
+    else if (kind == 3) k = hipMemcpyDeviceToDevice;
+    else return LLMI_ERR_INVALID_ARG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // A NULL stream copies synchronously, a stream asynchronously (alloc.cpp:28-46).
+    hipError_t err = s ? hipMemcpyAsync(dst, src, bytes, k, s) : hipMemcpy(dst, src, bytes, k);
+    if (err != hipSuccess) return record_hip_error(err, "hipMemcpy");
+    if (need_sync) return record_hip_error(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return LLMI_OK;
+}
+
+int llmi_hip_memset_zero(void* ptr, size_t bytes, void* stream, int32_t need_sync) {
+    if (!ptr) return LLMI_ERR_NULL_POINTER;
+    if (bytes == 0) return LLMI_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t err = s ? hipMemsetAsync(ptr, 0, bytes, s) : hipMemset(ptr, 0, bytes);  // alloc.cpp:61-66
+    if (err != hipSuccess) return record_hip_error(err, "hipMemset");
+    if (need_sync) return record_hip_error(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return LLMI_OK;
+}
+
+int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }
+
+const char* llmi_hip_strerror(int status) {
+    switch (status) {
+        case LLMI_OK: return "ok";
+        case LLMI_ERR_NULL_POINTER: return "required pointer is NULL";
+        case LLMI_ERR_HEAD_DIM: return "head_dim must be 128";
+        case LLMI_ERR_KV_DIM: return "kv_dim must be a positive multiple of head_dim";
+        case LLMI_ERR_ALIGNMENT: return "pointer is not sufficiently aligned (16 bytes for q/K/V/out/workspace)";
+        case LLMI_ERR_POS_RANGE: return "pos out of range [0, max_seq_len)";
+        case LLMI_ERR_WORKSPACE: return "split workspace missing or too small";
+        case LLMI_ERR_HEAD_GROUP: return "head_num must equal kv_mul * kv_heads with 1 <= kv_mul <= 16";
+        case LLMI_ERR_LAYOUT: return "unknown kv_layout";
+        case LLMI_ERR_INVALID_ARG: return "argument out of range";
+        case LLMI_ERR_LAUNCH: return "HIP call or kernel launch failed (see llmi_hip_last_error)";
+        case LLMI_ERR_UNKNOWN_POINTER: return "pointer is not a busy block of this pool";
+        case LLMI_ERR_OUT_OF_MEMORY: return "backing allocator failed";
+        default: return "unknown status";
+    }
+}
+
+const char* llmi_hip_last_error(void) { return g_last_error.c_str(); }
+
+}  // extern "C"

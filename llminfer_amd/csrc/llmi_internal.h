@@ -1,0 +1,30 @@
+// Internal declarations shared by the translation units of libllmi_hip.so.
+#ifndef LLMI_INTERNAL_H
+#define LLMI_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+
+#include "llmi_hip.h"
+
+namespace llmi {
+
+constexpr int kMaxSplits = 256;     // upper bound on the KV split count
+constexpr int kMaxGroup = 16;       // query heads per KV head the kernels accept
+constexpr int kMaxGroupWaves = 64;  // group_pad * waves_per_group that fits the LDS merge
+constexpr int kMaxWaves = 8;        // wavefronts per workgroup (512 threads keep 256 VGPRs per lane)
+
+// Records a failed HIP call for llmi_hip_last_error() and maps it to LLMI_ERR_LAUNCH.
+int record_hip_error(hipError_t err, const char* what);
+// hipGetLastError() after a kernel launch.
+int check_launch();
+
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan);
+int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);
+int launch_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,
+                        hipStream_t stream);
+int launch_kv_restride(const void* src, void* dst, int32_t layer_num, int32_t max_seq_len,
+                       int32_t kv_dim, int32_t head_dim, int32_t num_pos, hipStream_t stream);
+
+}  // namespace llmi
+
+#endif

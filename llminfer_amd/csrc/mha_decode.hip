@@ -1,0 +1,393 @@
+// Decode-phase grouped-query attention for gfx950 (MI355X), batch 1.
+//
+// One kernel template serves both paths of the reference's dispatcher
+// (code/source/op/kernel/cuda/mha_kernel.cu:505-528):
+//   * single pass  (num_splits == 1): the workgroup owns every position of one
+//     KV head and writes the bf16 result itself;
+//   * KV split     (num_splits  > 1): workgroup (split, kv_head) owns a
+//     contiguous range of positions and leaves (o[128], m, l) per query head
+//     in the fp32 workspace; mha_combine_kernel merges them (log-sum-exp).
+//
+// Differences from the reference design, chosen for CDNA4:
+//   * a workgroup serves ALL query heads of its KV head, so K and V are read
+//     from HBM exactly once (the reference re-reads them once per query head,
+//     mha_kernel.cu:67,104);
+//   * q.K^T runs on the matrix cores: one v_mfma_f32_16x16x32_bf16 chain per
+//     tile of 16 positions, K rows as the A operand straight from 16-byte
+//     global loads (lane = row, no LDS transpose needed because the
+//     contraction over head_dim is order-free), the query group as B;
+//   * p.V stays on the vector ALU in fp32 (p is never rounded to bf16): each
+//     16-lane DPP row owns 4 positions of the tile and 128 output columns,
+//     and picks its softmax weights out of the MFMA result layout with
+//     row_newbcast -- no LDS traffic in the inner loop;
+//   * running max / sum are kept in the exp2 domain (scale*log2(e) folded in);
+//   * 64-bit offsets throughout (the reference's int32 layer_offset,
+//     mha_kernel.cu:488, overflows on large caches).
+//
+// Tile bookkeeping (T = 16 consecutive positions, r = row in tile, h = head in group):
+//   MFMA A  lane L: row r = L%16, dims (j*4 + L/16)*8 .. +8 for step j = 0..3
+//   MFMA B  lane L: head h = L%16 (zero for h >= group), same dims
+//   MFMA C  lane L: head h = L%16, rows r = 4*(L/16) + i in register i = 0..3
+//   V / O   lane L: rows r = 4*(L/16) + i (load i), dims (L%16)*8 .. +8
+// so the weight of (row 4*(L/16)+i, head h) sits in lane (L/16)*16 + h,
+// register i: the same DPP row as every lane that needs it.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "llmi_internal.h"
+
+namespace llmi {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kTile = 16;      // positions per MFMA tile
+constexpr int kHeadDim = 128;
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// Value of lane SRC of the caller's 16-lane DPP row.
+template <int SRC>
+__device__ __forceinline__ float row_bcast(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + SRC, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// Round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if (x != x) return 0x7fc0;
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+struct TileRegs {
+    u32x4 k[4];
+    u32x4 v[4];
+};
+
+struct KernelArgs {
+    const uint16_t* q;    // [n_kv*group][128]
+    const uint16_t* k;    // layer base
+    const uint16_t* v;    // layer base
+    float* ws;            // split partials (num_splits > 1)
+    uint16_t* out;        // [n_kv*group][128]
+    float* out_f32;       // optional
+    int64_t row_stride;   // elements between consecutive positions of one KV head
+    int64_t head_stride;  // elements between KV heads
+    int32_t seq_len;
+    int32_t group;        // query heads per KV head
+    int32_t n_q;          // query heads
+    int32_t num_splits;
+    int32_t rows_per_split;  // multiple of kTile
+    float scale_log2e;       // log2(e) / sqrt(head_dim)
+};
+
+template <int G, int NW>
+__global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n16 = lane & 15;  // MFMA column / DPP-row lane
+    const int kg = lane >> 4;   // MFMA k-group / DPP row
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+
+    const int begin = split * a.rows_per_split;
+    const int end = min(begin + a.rows_per_split, a.seq_len);
+    const int last = end - 1;
+
+    // Query group as the MFMA B operand (zero columns beyond the group).
+    u32x4 qb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        u32x4 z = {0u, 0u, 0u, 0u};
+        if (n16 < a.group) {
+            const uint16_t* qp = a.q + ((int64_t)(kvh * a.group + n16) * kHeadDim + (j * 4 + kg) * 8);
+            z = *reinterpret_cast<const u32x4*>(qp);
+        }
+        qb[j] = z;
+    }
+
+    const uint16_t* kbase = a.k + (int64_t)kvh * a.head_stride + kg * 8;
+    const uint16_t* vbase = a.v + (int64_t)kvh * a.head_stride + n16 * 8;
+
+    float m_run = -INFINITY;  // running max, exp2 domain, per (head = n16)
+    float l_run = 0.0f;       // running sum over this lane's rows
+    float o[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[h][e] = 0.0f;
+
+    // Rows past the end of the range are clamped to its last row (a valid
+    // address) and masked out of the softmax below.
+    auto load_tile = [&](int t0, TileRegs& t) {
+        const int kr = min(t0 + n16, last);
+        const uint16_t* kp = kbase + (int64_t)kr * a.row_stride;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const u32x4*>(kp + j * 32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int vr = min(t0 + 4 * kg + i, last);
+            t.v[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)vr * a.row_stride);
+        }
+    };
+
+    auto compute_tile = [&](int t0, const TileRegs& t) {
+        f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.k[j]),
+                                                        __builtin_bit_cast(bf16x8, qb[j]), c, 0, 0, 0);
+        float s[4];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s[i] = (t0 + 4 * kg + i < end) ? c[i] * a.scale_log2e : -INFINITY;
+            tmax = fmaxf(tmax, s[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = fast_exp2(m_run - m_new);
+        float p[4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[i] = fast_exp2(s[i] - m_new);
+            psum += p[i];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+
+        // Rescale only when some head's max moved (wave-uniform test).
+        if (__any(alpha != 1.0f)) {
+            static_for<0, G>([&](auto h) {
+                const float ah = row_bcast<h.value>(alpha);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[h.value][e] *= ah;
+            });
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float vf[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                vf[2 * w] = bf16_lo(t.v[i][w]);
+                vf[2 * w + 1] = bf16_hi(t.v[i][w]);
+            }
+            static_for<0, G>([&](auto h) {
+                const float ph = row_bcast<h.value>(p[i]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[h.value][e] = __builtin_fmaf(ph, vf[e], o[h.value][e]);
+            });
+        }
+    };
+
+    // Two register sets, loads for the next tile in flight while the current one is consumed.
+    const int step = NW * kTile;
+    int t0 = begin + wave * kTile;
+    TileRegs ta, tb;
+    if (t0 < end) load_tile(t0, ta);
+    while (t0 < end) {
+        int tn = t0 + step;
+        if (tn < end) load_tile(tn, tb);
+        compute_tile(t0, ta);
+        t0 = tn;
+        if (t0 >= end) break;
+        tn = t0 + step;
+        if (tn < end) load_tile(tn, ta);
+        compute_tile(t0, tb);
+        t0 = tn;
+    }
+
+    // Fold the four DPP rows of the wave together (same head / same columns).
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float x = o[h][e];
+            x += __shfl_xor(x, 16);
+            x += __shfl_xor(x, 32);
+            o[h][e] = x;
+        }
+
+    // Merge the waves of the workgroup through LDS.
+    __shared__ float s_o[NW][G][kHeadDim];
+    __shared__ float s_m[NW][G];
+    __shared__ float s_l[NW][G];
+    if (kg == 0) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float* dst = &s_o[wave][h][n16 * 8];
+            *reinterpret_cast<f32x4*>(dst) = f32x4{o[h][0], o[h][1], o[h][2], o[h][3]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[h][4], o[h][5], o[h][6], o[h][7]};
+        }
+        if (n16 < G) {
+            s_m[wave][n16] = m_run;
+            s_l[wave][n16] = l_run;
+        }
+    }
+    __syncthreads();
+
+    const int n_out = a.group * kHeadDim;
+    for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
+        const int h = idx >> 7;
+        const int d = idx & (kHeadDim - 1);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) mx = fmaxf(mx, s_m[w][h]);
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float mw = s_m[w][h];
+            const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - mx);
+            acc += s_o[w][h][d] * f;
+            lsum += s_l[w][h] * f;
+        }
+        const int hq = kvh * a.group + h;
+        if (a.num_splits == 1) {
+            const float r = acc / lsum;
+            a.out[(int64_t)hq * kHeadDim + d] = f32_to_bf16(r);
+            if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
+        } else {
+            const int64_t S = a.num_splits;
+            a.ws[((int64_t)hq * S + split) * kHeadDim + d] = acc;
+            if (d == 0) {
+                a.ws[(int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split] = mx;
+                a.ws[(int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split] = lsum;
+            }
+        }
+    }
+}
+
+// Log-sum-exp merge of the split partials of one query head
+// (role of flashdecoding_gqa_combine_kernel, mha_kernel.cu:399-438).
+__global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __restrict__ ws,
+                                                                uint16_t* __restrict__ out,
+                                                                float* __restrict__ out_f32, int32_t n_q,
+                                                                int32_t num_splits) {
+    __shared__ float s_w[kMaxSplits];
+    __shared__ float s_red[2];
+    const int hq = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int64_t S = num_splits;
+    const float* ms = ws + (int64_t)n_q * S * kHeadDim + (int64_t)hq * S;
+    const float* ls = ws + (int64_t)n_q * S * (kHeadDim + 1) + (int64_t)hq * S;
+
+    float mx = -INFINITY;
+    for (int s = tid; s < num_splits; s += kHeadDim) mx = fmaxf(mx, ms[s]);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    if ((tid & 63) == 0) s_red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(s_red[0], s_red[1]);
+    __syncthreads();
+
+    float lsum = 0.0f;
+    for (int s = tid; s < num_splits; s += kHeadDim) {
+        const float m = ms[s];
+        const float f = (m == -INFINITY) ? 0.0f : fast_exp2(m - mx);
+        s_w[s] = f;
+        lsum += ls[s] * f;
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) lsum += __shfl_xor(lsum, d);
+    if ((tid & 63) == 0) s_red[tid >> 6] = lsum;
+    __syncthreads();
+    lsum = s_red[0] + s_red[1];
+
+    const float* os = ws + (int64_t)hq * S * kHeadDim + tid;
+    float acc = 0.0f;
+    for (int s = 0; s < num_splits; ++s) acc += os[(int64_t)s * kHeadDim] * s_w[s];
+    const float r = acc / lsum;
+    out[(int64_t)hq * kHeadDim + tid] = f32_to_bf16(r);
+    if (out_f32) out_f32[(int64_t)hq * kHeadDim + tid] = r;
+}
+
+template <int G, int NW>
+void launch_decode(const KernelArgs& ka, int n_kv, hipStream_t stream) {
+    dim3 grid(ka.num_splits, n_kv);
+    hipLaunchKernelGGL((mha_decode_kernel<G, NW>), grid, dim3(NW * 64), 0, stream, ka);
+}
+
+template <int G>
+bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream) {
+    switch (nw) {
+        case 1: launch_decode<G, 1>(ka, n_kv, stream); return true;
+        case 2: launch_decode<G, 2>(ka, n_kv, stream); return true;
+        case 4: launch_decode<G, 4>(ka, n_kv, stream); return true;
+        case 8:
+            if constexpr (G <= 8) { launch_decode<G, 8>(ka, n_kv, stream); return true; }
+            return false;
+        default: return false;
+    }
+}
+
+}  // namespace
+
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
+    const int n_kv = args.kv_dim / args.head_dim;
+    const int64_t layer_off = (int64_t)args.layer_id * args.max_seq_len * args.kv_dim;
+
+    KernelArgs ka;
+    ka.q = static_cast<const uint16_t*>(args.query);
+    ka.k = static_cast<const uint16_t*>(args.key_cache) + layer_off;
+    ka.v = static_cast<const uint16_t*>(args.value_cache) + layer_off;
+    ka.ws = static_cast<float*>(args.workspace);
+    ka.out = static_cast<uint16_t*>(args.output);
+    ka.out_f32 = args.output_f32;
+    if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
+        ka.row_stride = args.kv_dim;
+        ka.head_stride = args.head_dim;
+    } else {
+        ka.row_stride = args.head_dim;
+        ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
+    }
+    ka.seq_len = args.pos + 1;
+    ka.group = args.kv_mul;
+    ka.n_q = args.head_num;
+    ka.num_splits = plan.num_splits;
+    ka.rows_per_split = plan.rows_per_split;
+    ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
+
+    hipStream_t stream = static_cast<hipStream_t>(args.stream);
+    bool ok = false;
+    switch (plan.group_pad) {
+        case 1: ok = launch_decode_nw<1>(ka, n_kv, plan.waves_per_group, stream); break;
+        case 2: ok = launch_decode_nw<2>(ka, n_kv, plan.waves_per_group, stream); break;
+        case 4: ok = launch_decode_nw<4>(ka, n_kv, plan.waves_per_group, stream); break;
+        case 8: ok = launch_decode_nw<8>(ka, n_kv, plan.waves_per_group, stream); break;
+        case 16: ok = launch_decode_nw<16>(ka, n_kv, plan.waves_per_group, stream); break;
+        default: ok = false;
+    }
+    if (!ok) return LLMI_ERR_INVALID_ARG;
+    if (int rc = check_launch()) return rc;
+
+    if (plan.num_splits > 1) {
+        hipLaunchKernelGGL(mha_combine_kernel, dim3(args.head_num), dim3(kHeadDim), 0, stream, ka.ws, ka.out,
+                           ka.out_f32, args.head_num, plan.num_splits);
+        if (int rc = check_launch()) return rc;
+    }
+    return LLMI_OK;
+}
+
+}  // namespace llmi

@@ -1,0 +1,111 @@
+"""GPU parity of llmi_hip_mha_decode (through the C ABI) against the CPU oracle
+on the same seeded, bf16-rounded inputs. Gate: |d| <= 2e-3 + 1e-2*|ref| on the
+bf16 output, and max-abs <= 2e-3; the fp32 tap is held to a tighter bound."""
+import numpy as np
+import pytest
+
+from llminfer_amd import _binding as B
+from llminfer_amd import synth
+
+from helpers import assert_parity, assert_tap_parity, run_hip, run_oracle
+
+pytestmark = pytest.mark.gpu
+
+QWEN3_4B = dict(n_q=32, n_kv=8)
+
+
+def _check(oracle, dev, case, **kw):
+    ref = run_oracle(oracle, case)
+    got16, got32, plan = run_hip(case, dev, want_plan=True, **kw)
+    what = "ctx=%d path=%d splits=%d waves=%d %s" % (case["pos"] + 1, plan.path, plan.num_splits,
+                                                     plan.waves_per_group, kw)
+    assert_parity(got16, ref, "bf16 out " + what)
+    assert_tap_parity(got32, ref, what)
+    return plan
+
+
+@pytest.mark.parametrize("ctx", [128, 512, 1024, 2048])
+@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
+def test_qwen3_4b_short_context(oracle, dev, ctx, layout):
+    """Qwen3-4B layer shape, ctx 128..2048, seed 2, both cache layouts, dispatcher's choice."""
+    case = synth.make_case(2, ctx=ctx, **QWEN3_4B)
+    _check(oracle, dev, case, kv_layout=layout)
+
+
+@pytest.mark.parametrize("ctx", [128, 512, 1024, 2048])
+def test_single_pass_forced(oracle, dev, ctx):
+    case = synth.make_case(2, ctx=ctx, **QWEN3_4B)
+    plan = _check(oracle, dev, case, force_path=B.PATH_SINGLE_PASS)
+    assert plan.path == B.PATH_SINGLE_PASS and plan.num_splits == 1
+
+
+@pytest.mark.parametrize("ctx", [4096, 8192, 16384, 32768])
+def test_qwen3_4b_long_context(oracle, dev, ctx):
+    """Long-context KV-split path, seed 3, head-major layout (the production layout)."""
+    case = synth.make_case(3, ctx=ctx, **QWEN3_4B)
+    plan = _check(oracle, dev, case, kv_layout=B.KV_LAYOUT_HEAD_MAJOR)
+    assert plan.path == B.PATH_SPLIT and plan.num_splits > 1
+
+
+@pytest.mark.parametrize("splits", [2, 4, 8, 16, 32, 64, 256])
+@pytest.mark.parametrize("waves", [1, 2, 4, 8])
+def test_split_sweep_matches_oracle(oracle, dev, splits, waves):
+    """Any split count / workgroup shape gives the oracle's answer (ctx 4096)."""
+    case = synth.make_case(3, ctx=4096, **QWEN3_4B)
+    _check(oracle, dev, case, num_splits=splits, waves_per_group=waves, force_path=B.PATH_SPLIT)
+
+
+@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 1000, 4097])
+@pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT])
+def test_ragged_lengths(oracle, dev, ctx, path):
+    """Lengths around the 16-row tile, the wave count and the dispatch threshold; the cache rows past
+    pos hold NaN patterns, so any over-read shows."""
+    case = synth.make_case(100 + ctx, ctx=ctx, max_seq_len=ctx + 7, **QWEN3_4B)
+    _check(oracle, dev, case, force_path=path, num_splits=0 if path == B.PATH_SINGLE_PASS else 5)
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(8, 8), (16, 8), (32, 8), (64, 8), (6, 2), (12, 4), (16, 1), (20, 4)])
+@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
+def test_group_sizes_and_layers(oracle, dev, n_q, n_kv, layout):
+    """kv_mul 1..16 (incl. non powers of two), a non-zero layer of a multi-layer cache with
+    max_seq_len > seq_len: the shapes of the reference's own op test (test_op_mha.cpp:9-18,68-78)."""
+    case = synth.make_case(7, n_q=n_q, n_kv=n_kv, ctx=333, max_seq_len=400, layers=3, layer_id=2)
+    _check(oracle, dev, case, kv_layout=layout)
+    _check(oracle, dev, case, kv_layout=layout, force_path=B.PATH_SPLIT, num_splits=7)
+
+
+def test_unnormalised_inputs(oracle, dev):
+    """Plain N(0,1) inputs (no RMS normalisation): larger score spread, peaked softmax."""
+    case = synth.make_case(11, ctx=777, rms_norm=False, **QWEN3_4B)
+    case["q"] = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(case["q"]) * 3.0)
+    _check(oracle, dev, case)
+    _check(oracle, dev, case, force_path=B.PATH_SPLIT, num_splits=13)
+
+
+def test_qwen3_0p6b_layout_bf16(oracle, dev):
+    """16 Q / 8 KV heads, 256 cached + 1 new position (the CPU-plumbing shape, here in bf16)."""
+    case = synth.make_case(1, n_q=16, n_kv=8, ctx=257, max_seq_len=512, rms_norm=False)
+    _check(oracle, dev, case)
+
+
+def test_split_equals_single_pass(dev):
+    """Property at full size: split and single-pass agree on the fp32 tap (ctx 32768), no oracle needed."""
+    case = synth.make_case(5, ctx=32768, **QWEN3_4B)
+    _, one = run_hip(case, dev, force_path=B.PATH_SINGLE_PASS)
+    for splits in (4, 64, 256):
+        _, many = run_hip(case, dev, force_path=B.PATH_SPLIT, num_splits=splits)
+        assert np.all(np.abs(one - many) <= 1e-5 + 1e-4 * np.abs(one))
+
+
+def test_one_hot_attention(dev):
+    """One key far above the rest: the output is that position's V row exactly (bf16 values pass through)."""
+    case = synth.make_case(9, ctx=2000, **QWEN3_4B)
+    q = synth.bf16_bits_to_f32(case["q"]).reshape(32, 128)
+    k = case["k"]
+    target = 1234
+    for kvh in range(8):
+        # K[target] = 40 * mean of the group's queries: score ~ 40*|q|^2/sqrt(128) >> all others.
+        k[0, target, kvh * 128:(kvh + 1) * 128] = synth.f32_to_bf16_bits(40.0 * q[kvh * 4:(kvh + 1) * 4].mean(0))
+    got16, _ = run_hip(case, dev, force_path=B.PATH_SPLIT, num_splits=16)
+    want = synth.bf16_bits_to_f32(case["v"][0, target]).reshape(8, 1, 128).repeat(4, axis=1).reshape(-1)
+    assert np.allclose(got16, want, atol=2e-3, rtol=1e-2)
