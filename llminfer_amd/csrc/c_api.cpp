@@ -118,7 +118,7 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
             waves = a->waves_per_group;
         } else {
             waves = pow2_ceil(tiles);
-            if (waves > kMaxWaves) waves = kMaxWaves;
+            if (waves > kAutoMaxWaves) waves = kAutoMaxWaves;
             if (waves > max_waves) waves = max_waves;
         }
     }

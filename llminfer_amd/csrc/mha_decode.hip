@@ -50,6 +50,15 @@ namespace {
 constexpr int kTile = 16;      // positions per MFMA tile
 constexpr int kHeadDim = 128;
 
+// Build-time tuning knobs.
+#ifndef LLMI_NT_LOADS
+#define LLMI_NT_LOADS 1  // K/V are read once: stream them past the caches
+#endif
+#ifndef LLMI_MIN_WAVES_PER_EU
+#define LLMI_MIN_WAVES_PER_EU 2
+#endif
+
+
 template <int I, int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
     if constexpr (I < N) {
@@ -77,6 +86,27 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// 16 bytes per lane from global memory straight into LDS, no VGPR round trip:
+// lane L's bytes land at lds_off + 16*L. `base` and `lds_off` are wave-uniform,
+// `voff` is the lane's byte offset from base. Counted by vmcnt like any load.
+__device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t lds_off) {
+#if LLMI_NT_LOADS
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                 :: "s"(lds_off), "v"(voff), "s"(base) : "memory");
+#else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_off), "v"(voff), "s"(base) : "memory");
+#endif
+}
+
+// Waits until at most `newer_tiles` whole tiles (8 loads each) are still in flight.
+__device__ __forceinline__ void wait_tiles_in_flight(int newer_tiles) {
+    if (newer_tiles <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if (newer_tiles == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (newer_tiles == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+}
+
 struct TileRegs {
     u32x4 k[4];
     u32x4 v[4];
@@ -89,7 +119,7 @@ struct KernelArgs {
     float* ws;            // split partials (num_splits > 1)
     uint16_t* out;        // [n_kv*group][128]
     float* out_f32;       // optional
-    int64_t row_stride;   // elements between consecutive positions of one KV head
+    int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
     int32_t group;        // query heads per KV head
@@ -99,33 +129,44 @@ struct KernelArgs {
     float scale_log2e;       // log2(e) / sqrt(head_dim)
 };
 
-template <int G, int NW>
-__global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
+template <int G, int NW, int NSTAGE>
+__global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
     const int kg = lane >> 4;   // MFMA k-group / DPP row
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
 
     const int begin = split * a.rows_per_split;
-    const int end = min(begin + a.rows_per_split, a.seq_len);
-    const int last = end - 1;
+    const int nrows = min(a.rows_per_split, a.seq_len - begin);  // > 0: the host never makes empty splits
+    const int ntiles = (nrows + kTile - 1) / kTile;
 
-    // Query group as the MFMA B operand (zero columns beyond the group).
+    // Query group as the MFMA B operand (zero columns beyond the group). The
+    // load itself is unpredicated (padding lanes re-read the last head) so
+    // that it does not force a full wait on the first K/V tile.
     u32x4 qb[4];
+    {
+        const int hq = kvh * a.group + min(n16, a.group - 1);
+        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim + kg * 8;
+        const bool live = n16 < a.group;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        u32x4 z = {0u, 0u, 0u, 0u};
-        if (n16 < a.group) {
-            const uint16_t* qp = a.q + ((int64_t)(kvh * a.group + n16) * kHeadDim + (j * 4 + kg) * 8);
-            z = *reinterpret_cast<const u32x4*>(qp);
+        for (int j = 0; j < 4; ++j) {
+            const u32x4 z = *reinterpret_cast<const u32x4*>(qp + j * 32);
+            qb[j] = live ? z : u32x4{0u, 0u, 0u, 0u};
         }
-        qb[j] = z;
     }
 
-    const uint16_t* kbase = a.k + (int64_t)kvh * a.head_stride + kg * 8;
-    const uint16_t* vbase = a.v + (int64_t)kvh * a.head_stride + n16 * 8;
+    // Wave-uniform 64-bit bases of this split; lanes add 32-bit byte offsets
+    // (scalar-base + vector-offset addressing, no 64-bit multiplies per load).
+    const char* kb = reinterpret_cast<const char*>(a.k + (int64_t)kvh * a.head_stride + (int64_t)begin * a.row_stride);
+    const char* vb = reinterpret_cast<const char*>(a.v + (int64_t)kvh * a.head_stride + (int64_t)begin * a.row_stride);
+    const uint32_t rs = (uint32_t)a.row_stride * 2u;           // bytes per position step
+    const uint32_t last_off = (uint32_t)(nrows - 1) * rs;      // rows past the range clamp to its last row
+    const uint32_t k_row = (uint32_t)n16 * rs;
+    const uint32_t k_col = (uint32_t)kg * 16u;
+    const uint32_t v_row = (uint32_t)(4 * kg) * rs;
+    const uint32_t v_col = (uint32_t)n16 * 16u;
 
     float m_run = -INFINITY;  // running max, exp2 domain, per (head = n16)
     float l_run = 0.0f;       // running sum over this lane's rows
@@ -135,31 +176,54 @@ __global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[h][e] = 0.0f;
 
-    // Rows past the end of the range are clamped to its last row (a valid
-    // address) and masked out of the softmax below.
-    auto load_tile = [&](int t0, TileRegs& t) {
-        const int kr = min(t0 + n16, last);
-        const uint16_t* kp = kbase + (int64_t)kr * a.row_stride;
+    // Each wave streams its tiles through a private ring of NSTAGE LDS slots
+    // (8 KiB each: 4 KiB of K rows, 4 KiB of V rows) filled by LDS-DMA loads,
+    // so the bytes in flight cost no VGPRs. A lane later reads back exactly the
+    // 16 bytes it asked for (offset 16*lane inside each 1 KiB load), so the LDS
+    // reads are linear and conflict-free. Out-of-range rows of a ragged last
+    // tile read the last valid row and are masked out of the softmax.
+    constexpr int kStageBytes = 8192;
+    constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
+    constexpr int kMergeBytes = NW * G * (kHeadDim + 2) * (int)sizeof(float);
+    __shared__ __attribute__((aligned(1024))) char smem[kRingBytes > kMergeBytes ? kRingBytes : kMergeBytes];
+    char* my_ring = smem + wave * (NSTAGE * kStageBytes);
+    const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
+
+    auto issue_tile = [&](int t, int stage) {
+        // The slot's previous contents must have reached the VGPRs first.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const uint32_t base = (uint32_t)t * (kTile * rs);
+        const uint32_t slot = my_ring_lds + (uint32_t)stage * kStageBytes;
+        const uint32_t ko = min(base + k_row, last_off) + k_col;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) t.k[j] = *reinterpret_cast<const u32x4*>(kp + j * 32);
+        for (int j = 0; j < 4; ++j) dma16(kb, ko + j * 64, slot + j * 1024);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int vr = min(t0 + 4 * kg + i, last);
-            t.v[i] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)vr * a.row_stride);
+            const uint32_t vo = min(base + v_row + (uint32_t)i * rs, last_off) + v_col;
+            dma16(vb, vo, slot + 4096 + i * 1024);
         }
     };
 
-    auto compute_tile = [&](int t0, const TileRegs& t) {
+    auto read_tile = [&](int stage, TileRegs& r) {
+        const u32x4* sp = reinterpret_cast<const u32x4*>(my_ring + stage * kStageBytes) + lane;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r.k[j] = sp[j * 64];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.v[i] = sp[(4 + i) * 64];
+    };
+
+    auto compute_tile = [&](int t, const TileRegs& r) {
         f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.k[j]),
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, r.k[j]),
                                                         __builtin_bit_cast(bf16x8, qb[j]), c, 0, 0, 0);
+        const int row0 = t * kTile + 4 * kg;
         float s[4];
         float tmax = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            s[i] = (t0 + 4 * kg + i < end) ? c[i] * a.scale_log2e : -INFINITY;
+            s[i] = (row0 + i < nrows) ? c[i] * a.scale_log2e : -INFINITY;
             tmax = fmaxf(tmax, s[i]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
@@ -189,8 +253,8 @@ __global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
             float vf[8];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                vf[2 * w] = bf16_lo(t.v[i][w]);
-                vf[2 * w + 1] = bf16_hi(t.v[i][w]);
+                vf[2 * w] = bf16_lo(r.v[i][w]);
+                vf[2 * w + 1] = bf16_hi(r.v[i][w]);
             }
             static_for<0, G>([&](auto h) {
                 const float ph = row_bcast<h.value>(p[i]);
@@ -200,21 +264,19 @@ __global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
         }
     };
 
-    // Two register sets, loads for the next tile in flight while the current one is consumed.
-    const int step = NW * kTile;
-    int t0 = begin + wave * kTile;
-    TileRegs ta, tb;
-    if (t0 < end) load_tile(t0, ta);
-    while (t0 < end) {
-        int tn = t0 + step;
-        if (tn < end) load_tile(tn, tb);
-        compute_tile(t0, ta);
-        t0 = tn;
-        if (t0 >= end) break;
-        tn = t0 + step;
-        if (tn < end) load_tile(tn, ta);
-        compute_tile(t0, tb);
-        t0 = tn;
+    // Wave w owns tiles w, w+NW, ...: NSTAGE of them are always in flight.
+    const int n_my = wave < ntiles ? (ntiles - wave + NW - 1) / NW : 0;
+#pragma unroll
+    for (int s0 = 0; s0 < NSTAGE; ++s0)
+        if (s0 < n_my) issue_tile(wave + s0 * NW, s0);
+    int stage = 0;
+    for (int i = 0; i < n_my; ++i) {
+        TileRegs r;
+        wait_tiles_in_flight(min(NSTAGE - 1, n_my - 1 - i));
+        read_tile(stage, r);
+        if (i + NSTAGE < n_my) issue_tile(wave + (i + NSTAGE) * NW, stage);
+        compute_tile(wave + i * NW, r);
+        stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
     }
 
     // Fold the four DPP rows of the wave together (same head / same columns).
@@ -230,10 +292,14 @@ __global__ __launch_bounds__(NW * 64) void mha_decode_kernel(KernelArgs a) {
             o[h][e] = x;
         }
 
-    // Merge the waves of the workgroup through LDS.
-    __shared__ float s_o[NW][G][kHeadDim];
-    __shared__ float s_m[NW][G];
-    __shared__ float s_l[NW][G];
+    // Merge the waves of the workgroup through LDS (the ring is drained: every
+    // tile issued was waited for; reuse its memory once all waves are done with it).
+    __syncthreads();
+    typedef float (*MergeO)[G][kHeadDim];
+    typedef float (*MergeS)[G];
+    MergeO s_o = reinterpret_cast<MergeO>(smem);
+    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * G * kHeadDim * sizeof(float));
+    MergeS s_l = reinterpret_cast<MergeS>(smem + NW * G * (kHeadDim + 1) * sizeof(float));
     if (kg == 0) {
 #pragma unroll
         for (int h = 0; h < G; ++h) {
@@ -323,10 +389,16 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
     if (out_f32) out_f32[(int64_t)hq * kHeadDim + tid] = r;
 }
 
+#ifndef LLMI_STAGES
+#define LLMI_STAGES 2
+#endif
+
 template <int G, int NW>
 void launch_decode(const KernelArgs& ka, int n_kv, hipStream_t stream) {
+    // The LDS-DMA offset register addresses 64 KiB: NW * NSTAGE * 8 KiB must fit.
+    constexpr int kStages = (NW * LLMI_STAGES * 8192 <= 65536) ? LLMI_STAGES : 65536 / (NW * 8192);
     dim3 grid(ka.num_splits, n_kv);
-    hipLaunchKernelGGL((mha_decode_kernel<G, NW>), grid, dim3(NW * 64), 0, stream, ka);
+    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages>), grid, dim3(NW * 64), 0, stream, ka);
 }
 
 template <int G>
