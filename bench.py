@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ctx 1024,...,32768]
+
+One "step" is one layer call of llmi_hip_mha_decode (through the C ABI) at
+every context length of the sweep, Qwen3-4B layer shape (32 Q heads, 8 KV
+heads, head_dim 128), batch 1, bf16 KV cache in the head-major layout, inputs
+resident in HBM. Calls rotate over distinct slices of a KV arena much larger
+than the 256 MB Infinity Cache, so every call streams from HBM. The calls are
+captured into a HIP graph (no host code between kernels) and timed with HIP
+events on the stream that replays it.
+
+Prints ONE JSON line. `value` is algorithmic bytes per step / time per step.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_Q, N_KV, HEAD_DIM = 32, 8, 128
+KV_DIM = N_KV * HEAD_DIM
+HBM_PEAK_GBS = 8000.0
+DEFAULT_CTX = [1024, 2048, 4096, 8192, 16384, 32768]
+SLICES = 8  # distinct KV slices per context length inside one captured graph
+
+
+def algorithmic_bytes(ctx, n_q=N_Q, n_kv=N_KV):
+    """K and V rows once, q read once, out written once (bf16)."""
+    return 2 * ctx * n_kv * HEAD_DIM * 2 + 2 * n_q * HEAD_DIM * 2
+
+
+def make_arena(torch, dev, ctx_list):
+    """One K and one V slab; each (ctx, slice) pair owns a distinct region. Values: N(0,1),
+    RMS-normalised per 128-wide head vector, rounded to bf16."""
+    total_rows = sum(ctx_list) * SLICES
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(20260614)
+
+    def slab():
+        out = torch.empty((total_rows * N_KV, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+        chunk = 1 << 20
+        for lo in range(0, out.shape[0], chunk):
+            x = torch.randn((min(chunk, out.shape[0] - lo), HEAD_DIM), generator=gen, device=dev)
+            x = x * torch.rsqrt((x * x).mean(dim=1, keepdim=True))
+            out[lo:lo + chunk] = x.to(torch.bfloat16)
+        return out.reshape(-1)
+
+    k, v = slab(), slab()
+    regions = {}
+    row = 0
+    for ctx in ctx_list:
+        for s in range(SLICES):
+            regions[(ctx, s)] = row * KV_DIM  # element offset of a [N_KV][ctx][128] cache
+            row += ctx
+    q = torch.randn((N_Q, HEAD_DIM), generator=gen, device=dev)
+    q = (q * torch.rsqrt((q * q).mean(dim=1, keepdim=True))).to(torch.bfloat16).reshape(-1)
+    return k, v, q, regions
+
+
+def cpu_baseline(ctx_list, budget_s=12.0):
+    """The CPU oracle (a port of the reference's single-threaded CPU attention path) timed on this
+    host on the same shapes: whole sweeps until about `budget_s` seconds have been spent."""
+    import numpy as np
+    import oracle
+    from llminfer_amd import synth
+    cases = []
+    for ctx in ctx_list:
+        c = synth.make_case(1000 + ctx, n_q=N_Q, n_kv=N_KV, ctx=ctx)
+        cases.append(c)
+    oracle.lib()
+    passes, t_total = 0, 0.0
+    while t_total < budget_s and passes < 50:
+        t0 = time.perf_counter()
+        for c in cases:
+            oracle.mha_cpu(c["q"], c["k"], c["v"], c["layer_id"], c["pos"], c["kv_dim"], c["kv_mul"],
+                           c["head_num"], c["head_dim"], c["max_seq_len"])
+        t_total += time.perf_counter() - t0
+        passes += 1
+    nbytes = sum(algorithmic_bytes(c) for c in ctx_list) * passes
+    return {
+        "value": round(nbytes / t_total / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "%d passes of the same ctx sweep %s through the CPU oracle (bf16 inputs widened to fp32), "
+                  "%.1f s, %.0f us per layer call on average"
+                  % (passes, ctx_list, t_total, t_total / (passes * len(ctx_list)) * 1e6),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--ctx", type=str, default=",".join(map(str, DEFAULT_CTX)))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus %d refused): the path has no multi-GPU "
+              "part; see DESIGN.md for how it would shard." % args.gpus, file=sys.stderr)
+        return 2
+    ctx_list = [int(c) for c in args.ctx.split(",")]
+
+    import torch
+    from llminfer_amd import _binding as B
+    from llminfer_amd import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    B.lib()  # fail loudly if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    k, v, q, regions = make_arena(torch, dev, ctx_list)
+    out = torch.empty(N_Q * HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(ops.workspace_bytes(N_Q, HEAD_DIM, max(ctx_list)) // 4, dtype=torch.float32, device=dev)
+    esz = 2
+
+    def call_args(ctx, s):
+        off = regions[(ctx, s)] * esz
+        return ops.make_mha_args(q, k.data_ptr() + off, v.data_ptr() + off, out, ws, layer_id=0, pos=ctx - 1,
+                                 kv_dim=KV_DIM, kv_mul=N_Q // N_KV, head_num=N_Q, head_dim=HEAD_DIM,
+                                 max_seq_len=ctx, kv_layout=args.layout)
+
+    plans = {ctx: ops.mha_plan(call_args(ctx, 0)) for ctx in ctx_list}
+    stream = torch.cuda.Stream()
+    decode = B.lib().llmi_hip_mha_decode
+
+    def enqueue(ctxs, steps):
+        for s in range(steps):
+            for ctx in ctxs:
+                a = call_args(ctx, s % SLICES)
+                a.stream = stream.cuda_stream
+                B.check(decode(ctypes.byref(a)), "llmi_hip_mha_decode")
+
+    def capture(ctxs):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            enqueue(ctxs, 1)  # eager once: loads the code objects before capture
+            stream.synchronize()
+            with torch.cuda.graph(g, stream=stream):
+                enqueue(ctxs, SLICES)
+        return g
+
+    def time_graph(g, replays):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            e0.record(stream)
+            for _ in range(replays):
+                g.replay()
+            e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1)  # ms
+
+    # ---- the timed region: K steps of the whole sweep ----------------------
+    steps = max(SLICES, (args.steps + SLICES - 1) // SLICES * SLICES)
+    warm = max(SLICES, (args.warmup + SLICES - 1) // SLICES * SLICES)
+    g_all = capture(ctx_list)
+    time_graph(g_all, warm // SLICES)
+    torch.cuda.synchronize()
+    ms = time_graph(g_all, steps // SLICES)
+    torch.cuda.synchronize()
+    ms_per_step = ms / steps
+    step_bytes = sum(algorithmic_bytes(c) for c in ctx_list)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launches_per_step = len(ctx_list)  # every call of the sweep is one launch of the decode kernel
+
+    # ---- per-context figures (same method, one context at a time) ----------
+    per_ctx = []
+    for ctx in ctx_list:
+        g = capture([ctx])
+        time_graph(g, max(1, warm // SLICES))
+        torch.cuda.synchronize()
+        n = max(SLICES, steps)
+        t = time_graph(g, n // SLICES)
+        torch.cuda.synchronize()
+        us = t * 1e3 / n
+        gbs = algorithmic_bytes(ctx) / (us * 1e-6) / 1e9
+        p = plans[ctx]
+        per_ctx.append({"ctx": ctx, "us_per_layer": round(us, 3), "GBps": round(gbs, 1),
+                        "frac_peak": round(gbs / HBM_PEAK_GBS, 4), "path": p.path, "splits": p.num_splits,
+                        "waves": p.waves_per_group})
+
+    avg_launch_us = ms_per_step * 1e3 / launches_per_step
+    avg_launch_bytes = step_bytes / launches_per_step
+    achieved = avg_launch_bytes / (avg_launch_us * 1e-6) / 1e9
+    result = {
+        "metric": "GQA decode attn us/layer + HBM GB/s (% peak), Qwen3-4B shape, ctx 1K-32K",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Qwen3-4B layer shape (32 Q / 8 KV heads, head_dim 128), batch 1, one decode-"
+                               "attention layer call per context in %s per step, bf16 KV cache, %s layout, "
+                               "HIP-graph replays over %d rotating KV slices per context"
+                               % (ctx_list, "head-major" if args.layout == 1 else "position-major", SLICES),
+                   "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout},
+        "us_per_layer_mean": round(avg_launch_us, 3),
+        "per_ctx": per_ctx,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "mha_decode_kernel", "launches": steps * launches_per_step,
+                     "avg_launch_us": round(avg_launch_us, 3), "avg_launch_bytes": int(avg_launch_bytes)},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(ctx_list)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -66,7 +66,9 @@ enum {
     LLMI_KV_LAYOUT_HEAD_MAJOR = 1
 };
 
-enum { LLMI_PATH_AUTO = 0, LLMI_PATH_SINGLE_PASS = 1, LLMI_PATH_SPLIT = 2 };
+/* SPLIT runs the split kernel and then a combine kernel; SPLIT_FUSED runs the
+ * split kernel alone, whose last-arriving workgroup per KV head does the combine. */
+enum { LLMI_PATH_AUTO = 0, LLMI_PATH_SINGLE_PASS = 1, LLMI_PATH_SPLIT = 2, LLMI_PATH_SPLIT_FUSED = 3 };
 
 typedef struct llmi_mha_args {
     const void* query;        /* device, bf16 [head_num*head_dim]                        */
@@ -92,7 +94,7 @@ typedef struct llmi_mha_args {
 } llmi_mha_args;
 
 typedef struct llmi_mha_plan {
-    int32_t path;             /* LLMI_PATH_SINGLE_PASS or LLMI_PATH_SPLIT                */
+    int32_t path;             /* LLMI_PATH_SINGLE_PASS, LLMI_PATH_SPLIT or LLMI_PATH_SPLIT_FUSED */
     int32_t num_splits;       /* 1 for single-pass                                       */
     int32_t rows_per_split;   /* multiple of 16                                          */
     int32_t waves_per_group;
@@ -106,8 +108,10 @@ int llmi_hip_mha_plan(const llmi_mha_args* args, llmi_mha_plan* plan);
 
 /* Decode attention for one layer and one new token: for every query head h,
  * out[h] = softmax(q[h].K[h/kv_mul]^T / sqrt(128)) . V[h/kv_mul] over positions
- * 0..pos, bf16 in, fp32 accumulate, bf16 out. Enqueues 1 kernel (single-pass)
- * or 2 (split + combine). Allocates nothing; safe under stream capture. */
+ * 0..pos, bf16 in, fp32 accumulate, bf16 out. Enqueues 1 kernel (single-pass,
+ * split with fused combine) or 2 (split + combine). Allocates nothing; safe
+ * under stream capture. The workspace needs no initialisation. Two calls that
+ * share a workspace must not overlap in time. */
 int llmi_hip_mha_decode(const llmi_mha_args* args);
 
 /* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */

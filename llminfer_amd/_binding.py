@@ -13,7 +13,7 @@ c_size_t = ctypes.c_size_t
 LLMI_OK = 0
 KV_LAYOUT_POS_MAJOR = 0
 KV_LAYOUT_HEAD_MAJOR = 1
-PATH_AUTO, PATH_SINGLE_PASS, PATH_SPLIT = 0, 1, 2
+PATH_AUTO, PATH_SINGLE_PASS, PATH_SPLIT, PATH_SPLIT_FUSED = 0, 1, 2, 3
 
 STATUS = {
     "OK": 0, "NULL_POINTER": -1, "HEAD_DIM": -2, "KV_DIM": -3, "ALIGNMENT": -4, "POS_RANGE": -5,

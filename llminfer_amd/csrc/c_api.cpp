@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -22,8 +24,10 @@ thread_local std::string g_last_error;
 // splits, mha_kernel.cu:507-517; here a split costs a second launch and a
 // workspace round trip, and one workgroup already streams a whole KV head.)
 constexpr int kSinglePassMaxLen = 256;
-// Workgroups the split path aims for: a few per CU so every CU has loads in flight.
-constexpr int kTargetGroups = 1024;
+// Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
+// waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
+// add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).
+constexpr int kTargetGroups = 256;
 constexpr int kTile = 16;
 
 inline int pow2_ceil(int x) {
@@ -46,6 +50,18 @@ int record_hip_error(hipError_t err, const char* what) {
     return LLMI_ERR_LAUNCH;
 }
 
+unsigned long long next_epoch() {
+    // Starts from the clock so that a stale cell left in a reused workspace by
+    // another process run does not match; 48 bits, never 0.
+    static std::atomic<unsigned long long> counter{
+        (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count()};
+    unsigned long long e;
+    do {
+        e = counter.fetch_add(1, std::memory_order_relaxed) & 0xffffffffffffull;
+    } while (e == 0);
+    return e;
+}
+
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
 
 static int validate_mha(const llmi_mha_args* a) {
@@ -63,7 +79,7 @@ static int validate_mha(const llmi_mha_args* a) {
         return LLMI_ERR_ALIGNMENT;                                                  // mha_kernel.cu:495-498
     if (a->workspace && !aligned16(a->workspace)) return LLMI_ERR_ALIGNMENT;
     if (a->output_f32 && (reinterpret_cast<uintptr_t>(a->output_f32) & 3u)) return LLMI_ERR_ALIGNMENT;
-    if (a->force_path < LLMI_PATH_AUTO || a->force_path > LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
+    if (a->force_path < LLMI_PATH_AUTO || a->force_path > LLMI_PATH_SPLIT_FUSED) return LLMI_ERR_INVALID_ARG;
     if (a->num_splits < 0 || a->num_splits > kMaxSplits) return LLMI_ERR_INVALID_ARG;
     const int w = a->waves_per_group;
     if (!(w == 0 || w == 1 || w == 2 || w == 4 || w == 8)) return LLMI_ERR_INVALID_ARG;
@@ -79,17 +95,21 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
     int max_waves = pow2_floor(kMaxGroupWaves / group_pad);
     if (max_waves > kMaxWaves) max_waves = kMaxWaves;
     if (a->waves_per_group > max_waves) return LLMI_ERR_INVALID_ARG;
-    const size_t per_split = (size_t)a->head_num * (a->head_dim + 2) * sizeof(float);
+    const size_t per_split_plain = (size_t)a->head_num * (a->head_dim + 2) * sizeof(float);
+    const size_t per_split_fused = per_split_plain + (size_t)n_kv * sizeof(unsigned long long);
 
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
         else if (a->num_splits > 1) path = LLMI_PATH_SPLIT;
-        else path = seq_len <= kSinglePassMaxLen ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT;
+        else path = seq_len <= kSinglePassMaxLen ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT_FUSED;
+        if (path == LLMI_PATH_SPLIT) path = LLMI_PATH_SPLIT_FUSED;
     }
 
     int num_splits = 1, tiles_per_split = tiles, waves;
-    if (path == LLMI_PATH_SPLIT) {
+    if (path != LLMI_PATH_SINGLE_PASS) {
+        // The fused combine keeps one 8-byte arrival flag per (KV head, split) behind the partials.
+        const bool fused = path == LLMI_PATH_SPLIT_FUSED;
         waves = a->waves_per_group ? a->waves_per_group : (max_waves < 4 ? max_waves : 4);
         int want = a->num_splits;
         if (want == 0) {
@@ -98,7 +118,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
             want = kTargetGroups / n_kv;
             if (want < 2) want = 2;
             if (want > kMaxSplits) want = kMaxSplits;
-            const size_t cap = a->workspace ? a->workspace_bytes / per_split : 0;
+            const size_t per_split = fused ? per_split_fused : per_split_plain;
+            const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
             if (cap < 2) return LLMI_ERR_WORKSPACE;
             if ((size_t)want > cap) want = (int)cap;
             tiles_per_split = ceil_div(tiles, want);
@@ -108,7 +129,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
         }
         num_splits = ceil_div(tiles, tiles_per_split);  // no empty splits
         if (num_splits > 1) {
-            if (!a->workspace || a->workspace_bytes < per_split * (size_t)num_splits) return LLMI_ERR_WORKSPACE;
+            const size_t need = (fused ? per_split_fused : per_split_plain) * (size_t)num_splits + (fused ? 16 : 0);
+            if (!a->workspace || a->workspace_bytes < need) return LLMI_ERR_WORKSPACE;
         }
     }
     if (num_splits == 1) {
@@ -128,7 +150,9 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
     p->rows_per_split = tiles_per_split * kTile;
     p->waves_per_group = waves;
     p->group_pad = group_pad;
-    p->workspace_needed = num_splits > 1 ? per_split * (size_t)num_splits : 0;
+    p->workspace_needed = num_splits <= 1 ? 0
+                          : path == LLMI_PATH_SPLIT_FUSED ? per_split_fused * (size_t)num_splits + 16
+                                                          : per_split_plain * (size_t)num_splits;
     return LLMI_OK;
 }
 
@@ -153,7 +177,9 @@ size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t 
     if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     int splits = (max_seq_len + kTile - 1) / kTile;
     if (splits > kMaxSplits) splits = kMaxSplits;
-    return (size_t)head_num * (size_t)splits * (size_t)(head_dim + 2) * sizeof(float);
+    // Partials for the largest split count plus the arrival flags of the fused combine
+    // (one per KV head and split; head_num bounds the KV head count).
+    return (size_t)head_num * (size_t)splits * ((size_t)(head_dim + 2) * sizeof(float) + sizeof(unsigned long long)) + 16;
 }
 
 int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {

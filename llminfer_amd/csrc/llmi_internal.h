@@ -19,6 +19,9 @@ int record_hip_error(hipError_t err, const char* what);
 // hipGetLastError() after a kernel launch.
 int check_launch();
 
+// A fresh 48-bit tag per decode call (never 0), for the arrival cells of the fused combine.
+unsigned long long next_epoch();
+
 int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan);
 int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);
 int launch_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,

@@ -49,6 +49,9 @@ namespace {
 
 constexpr int kTile = 16;      // positions per MFMA tile
 constexpr int kHeadDim = 128;
+// Polls (each followed by a short sleep) the fused combine waits for the other splits: far
+// beyond any real kernel time, yet finite.
+constexpr int kMaxSpins = 1 << 22;
 
 // Build-time tuning knobs.
 #ifndef LLMI_NT_LOADS
@@ -119,6 +122,8 @@ struct KernelArgs {
     float* ws;            // split partials (num_splits > 1)
     uint16_t* out;        // [n_kv*group][128]
     float* out_f32;       // optional
+    unsigned long long* arrivals;  // [n_kv][num_splits] arrival flags of the fused combine, or nullptr
+    unsigned long long epoch;      // tag of this call, 48 bits
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
@@ -185,7 +190,10 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int kStageBytes = 8192;
     constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
     constexpr int kMergeBytes = NW * G * (kHeadDim + 2) * (int)sizeof(float);
-    __shared__ __attribute__((aligned(1024))) char smem[kRingBytes > kMergeBytes ? kRingBytes : kMergeBytes];
+    constexpr int kCombineBytes = (G * kMaxSplits + G) * (int)sizeof(float);
+    constexpr int kSmemBytes = kRingBytes > kMergeBytes ? (kRingBytes > kCombineBytes ? kRingBytes : kCombineBytes)
+                                                        : (kMergeBytes > kCombineBytes ? kMergeBytes : kCombineBytes);
+    __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * (NSTAGE * kStageBytes);
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
 
@@ -336,12 +344,110 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
             if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
         } else {
             const int64_t S = a.num_splits;
-            a.ws[((int64_t)hq * S + split) * kHeadDim + d] = acc;
-            if (d == 0) {
-                a.ws[(int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split] = mx;
-                a.ws[(int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split] = lsum;
+            float* po = a.ws + ((int64_t)hq * S + split) * kHeadDim + d;
+            float* pm = a.ws + (int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split;
+            float* pl = a.ws + (int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split;
+            if (a.arrivals) {
+                // Device-coherent stores: they go past this XCD's L2, so the
+                // workgroup (possibly on another XCD) that does the combine can
+                // read them without anyone flushing or invalidating a cache.
+                __hip_atomic_store(po, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (d == 0) {
+                    __hip_atomic_store(pm, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(pl, lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else {
+                *po = acc;
+                if (d == 0) {
+                    *pm = mx;
+                    *pl = lsum;
+                }
             }
         }
+    }
+
+    // Fused combine: the workgroup of the LAST split of this KV head merges the
+    // partials of its query heads, so no second launch is needed. Every split
+    // publishes a flag after its partials; the last split's workgroup waits for
+    // all flags. Workgroups are dispatched in index order and the others never
+    // wait for anything, so whoever it waits for is already running or done.
+    if (a.num_splits == 1 || a.arrivals == nullptr) return;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
+    __syncthreads();
+    // A flag holds the epoch of the call that set it; anything else (an
+    // uninitialised workspace, an earlier call) reads as "not arrived", so the
+    // workspace needs no clearing. The combiner zeroes the flags again so that
+    // a graph replay of this very call (same epoch) starts clean.
+    unsigned long long* flags = a.arrivals + (int64_t)kvh * a.num_splits;
+    if (split != a.num_splits - 1) {
+        if (threadIdx.x == 0) __hip_atomic_store(flags + split, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    __shared__ int s_all_arrived;
+    if (wave == 0) {
+        bool ok = false;
+        // Bounded wait: every wave leaves this loop even if a flag never shows up
+        // (the result is then marked invalid below instead of hanging the GPU).
+        for (int spin = 0; spin < kMaxSpins; ++spin) {
+            ok = true;
+            for (int sp = lane; sp < a.num_splits - 1; sp += 64)
+                ok = ok && (__hip_atomic_load(flags + sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch);
+            if (__all(ok)) break;
+            __builtin_amdgcn_s_sleep(8);
+        }
+        for (int sp = lane; sp < a.num_splits - 1; sp += 64)
+            __hip_atomic_store(flags + sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) s_all_arrived = __all(ok) ? 1 : 0;
+    }
+    __syncthreads();
+    const bool all_arrived = s_all_arrived != 0;
+    // Every other workgroup's partials were acknowledged before its flag was
+    // set; read them with device-coherent loads.
+    auto coherent = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+
+    float* s_w = reinterpret_cast<float*>(smem);                                   // [G][kMaxSplits] weights
+    float* s_den = reinterpret_cast<float*>(smem + G * kMaxSplits * sizeof(float));  // [G] denominators
+    const int S = a.num_splits;
+    const float* ws_m = a.ws + (int64_t)a.n_q * S * kHeadDim;
+    const float* ws_l = a.ws + (int64_t)a.n_q * S * (kHeadDim + 1);
+    // One wave per head: M = max m_s, weights e^(m_s - M), denominator sum l_s * weight.
+    for (int h = wave; h < a.group; h += NW) {
+        const int64_t row = (int64_t)(kvh * a.group + h) * S;
+        float mx = -INFINITY;
+        for (int sp = lane; sp < S; sp += 64) mx = fmaxf(mx, coherent(ws_m + row + sp));
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+        float den = 0.0f;
+        for (int sp = lane; sp < S; sp += 64) {
+            const float m = coherent(ws_m + row + sp);
+            const float f = (m == -INFINITY) ? 0.0f : fast_exp2(m - mx);
+            s_w[h * kMaxSplits + sp] = f;
+            den += coherent(ws_l + row + sp) * f;
+        }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) den += __shfl_xor(den, d);
+        if (lane == 0) s_den[h] = den;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
+        const int h = idx >> 7;
+        const int d = idx & (kHeadDim - 1);
+        const int hq = kvh * a.group + h;
+        const float* os = a.ws + (int64_t)hq * S * kHeadDim + d;
+        const float* w = s_w + h * kMaxSplits;
+        float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
+        int sp = 0;
+        for (; sp + 4 <= S; sp += 4) {
+            acc0 += coherent(os + (int64_t)(sp + 0) * kHeadDim) * w[sp + 0];
+            acc1 += coherent(os + (int64_t)(sp + 1) * kHeadDim) * w[sp + 1];
+            acc2 += coherent(os + (int64_t)(sp + 2) * kHeadDim) * w[sp + 2];
+            acc3 += coherent(os + (int64_t)(sp + 3) * kHeadDim) * w[sp + 3];
+        }
+        for (; sp < S; ++sp) acc0 += coherent(os + (int64_t)sp * kHeadDim) * w[sp];
+        // A wait that ran out of patience poisons the output rather than returning a partial sum.
+        const float r = all_arrived ? ((acc0 + acc1) + (acc2 + acc3)) / s_den[h] : __builtin_nanf("");
+        a.out[(int64_t)hq * kHeadDim + d] = f32_to_bf16(r);
+        if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
     }
 }
 
@@ -427,6 +533,15 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
     ka.ws = static_cast<float*>(args.workspace);
     ka.out = static_cast<uint16_t*>(args.output);
     ka.out_f32 = args.output_f32;
+    ka.arrivals = nullptr;
+    ka.epoch = 0;
+    if (plan.path == LLMI_PATH_SPLIT_FUSED) {
+        // Arrival flags sit behind the partials in the workspace.
+        const size_t partial_bytes = (size_t)args.head_num * plan.num_splits * (args.head_dim + 2) * sizeof(float);
+        ka.arrivals = reinterpret_cast<unsigned long long*>(static_cast<char*>(args.workspace) +
+                                                            ((partial_bytes + 15) & ~(size_t)15));
+        ka.epoch = next_epoch();
+    }
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
         ka.row_stride = args.kv_dim;
         ka.head_stride = args.head_dim;
@@ -454,7 +569,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
     if (!ok) return LLMI_ERR_INVALID_ARG;
     if (int rc = check_launch()) return rc;
 
-    if (plan.num_splits > 1) {
+    if (plan.num_splits > 1 && plan.path != LLMI_PATH_SPLIT_FUSED) {
         hipLaunchKernelGGL(mha_combine_kernel, dim3(args.head_num), dim3(kHeadDim), 0, stream, ka.ws, ka.out,
                            ka.out_f32, args.head_num, plan.num_splits);
         if (int rc = check_launch()) return rc;

@@ -44,19 +44,21 @@ def test_qwen3_4b_long_context(oracle, dev, ctx):
     """Long-context KV-split path, seed 3, head-major layout (the production layout)."""
     case = synth.make_case(3, ctx=ctx, **QWEN3_4B)
     plan = _check(oracle, dev, case, kv_layout=B.KV_LAYOUT_HEAD_MAJOR)
-    assert plan.path == B.PATH_SPLIT and plan.num_splits > 1
+    assert plan.path == B.PATH_SPLIT_FUSED and plan.num_splits > 1
 
 
 @pytest.mark.parametrize("splits", [2, 4, 8, 16, 32, 64, 256])
 @pytest.mark.parametrize("waves", [1, 2, 4, 8])
-def test_split_sweep_matches_oracle(oracle, dev, splits, waves):
-    """Any split count / workgroup shape gives the oracle's answer (ctx 4096)."""
+@pytest.mark.parametrize("path", [B.PATH_SPLIT, B.PATH_SPLIT_FUSED])
+def test_split_sweep_matches_oracle(oracle, dev, splits, waves, path):
+    """Any split count / workgroup shape gives the oracle's answer (ctx 4096), with the separate
+    combine kernel and with the combine fused into the split kernel's last-arriving workgroup."""
     case = synth.make_case(3, ctx=4096, **QWEN3_4B)
-    _check(oracle, dev, case, num_splits=splits, waves_per_group=waves, force_path=B.PATH_SPLIT)
+    _check(oracle, dev, case, num_splits=splits, waves_per_group=waves, force_path=path)
 
 
 @pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 1000, 4097])
-@pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT])
+@pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT, B.PATH_SPLIT_FUSED])
 def test_ragged_lengths(oracle, dev, ctx, path):
     """Lengths around the 16-row tile, the wave count and the dispatch threshold; the cache rows past
     pos hold NaN patterns, so any over-read shows."""
@@ -72,6 +74,7 @@ def test_group_sizes_and_layers(oracle, dev, n_q, n_kv, layout):
     case = synth.make_case(7, n_q=n_q, n_kv=n_kv, ctx=333, max_seq_len=400, layers=3, layer_id=2)
     _check(oracle, dev, case, kv_layout=layout)
     _check(oracle, dev, case, kv_layout=layout, force_path=B.PATH_SPLIT, num_splits=7)
+    _check(oracle, dev, case, kv_layout=layout, force_path=B.PATH_SPLIT_FUSED, num_splits=7)
 
 
 def test_unnormalised_inputs(oracle, dev):
@@ -92,9 +95,10 @@ def test_split_equals_single_pass(dev):
     """Property at full size: split and single-pass agree on the fp32 tap (ctx 32768), no oracle needed."""
     case = synth.make_case(5, ctx=32768, **QWEN3_4B)
     _, one = run_hip(case, dev, force_path=B.PATH_SINGLE_PASS)
-    for splits in (4, 64, 256):
-        _, many = run_hip(case, dev, force_path=B.PATH_SPLIT, num_splits=splits)
-        assert np.all(np.abs(one - many) <= 1e-5 + 1e-4 * np.abs(one))
+    for path in (B.PATH_SPLIT, B.PATH_SPLIT_FUSED):
+        for splits in (4, 64, 256):
+            _, many = run_hip(case, dev, force_path=path, num_splits=splits)
+            assert np.all(np.abs(one - many) <= 1e-5 + 1e-4 * np.abs(one))
 
 
 def test_one_hot_attention(dev):
@@ -109,3 +113,55 @@ def test_one_hot_attention(dev):
     got16, _ = run_hip(case, dev, force_path=B.PATH_SPLIT, num_splits=16)
     want = synth.bf16_bits_to_f32(case["v"][0, target]).reshape(8, 1, 128).repeat(4, axis=1).reshape(-1)
     assert np.allclose(got16, want, atol=2e-3, rtol=1e-2)
+
+
+def test_fused_combine_repeated_calls_share_workspace(oracle, dev):
+    """The arrival cells of the fused combine need no clearing: back-to-back calls on one workspace
+    (first full of NaN patterns), with different split counts and contexts, all match the oracle."""
+    import torch
+    from llminfer_amd import ops
+    from helpers import from_dev_bf16, to_dev
+    ws = torch.full((ops.workspace_bytes(32, 128, 4096) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    for seed, ctx, splits in [(21, 4096, 64), (22, 3000, 64), (23, 4096, 17), (24, 700, 0), (25, 4096, 64)]:
+        case = synth.make_case(seed, ctx=ctx, max_seq_len=4096, **QWEN3_4B)
+        ref = run_oracle(oracle, case)
+        q, k, v = to_dev(case["q"], dev), to_dev(case["k"], dev), to_dev(case["v"], dev)
+        out = torch.zeros(32 * 128, dtype=torch.int16, device=dev)
+        for _ in range(3):
+            ops.mha_decode(q, k, v, out, ws, layer_id=0, pos=ctx - 1, kv_dim=1024, kv_mul=4, head_num=32,
+                           head_dim=128, max_seq_len=4096, force_path=B.PATH_SPLIT_FUSED, num_splits=splits)
+        torch.cuda.synchronize()
+        assert_parity(from_dev_bf16(out), ref, "ctx=%d splits=%d" % (ctx, splits))
+
+
+def test_graph_replay_matches_eager(oracle, dev):
+    """A captured decode call (fused combine) replayed several times, with eager work and
+    synchronisation between the replays, gives the eager result every time."""
+    import torch
+    from llminfer_amd import ops
+    from helpers import from_dev_bf16, to_dev
+    case = synth.make_case(31, ctx=5000, **QWEN3_4B)
+    ref = run_oracle(oracle, case)
+    q, k, v = to_dev(case["q"], dev), to_dev(case["k"], dev), to_dev(case["v"], dev)
+    ws = torch.full((ops.workspace_bytes(32, 128, 5000) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    out = torch.zeros(32 * 128, dtype=torch.int16, device=dev)
+    kw = dict(layer_id=0, pos=4999, kv_dim=1024, kv_mul=4, head_num=32, head_dim=128, max_seq_len=5000)
+    ops.mha_decode(q, k, v, out, ws, **kw)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    assert_parity(from_dev_bf16(eager), ref, "eager")
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.mha_decode(q, k, v, out, ws, stream=side, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(4):
+        out.fill_(0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        scratch = torch.randn(1 << 16, device=dev).sum().item()  # unrelated eager work between replays
+        assert scratch == scratch
