@@ -1,0 +1,187 @@
+"""The C ABI without a GPU: the library loads, exports every symbol include/llmi_hip.h declares, its
+structs have the layout the binding assumes, and validation / dispatch planning (which make no HIP call)
+return the documented status codes."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from llminfer_amd import _binding as B
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "llmi_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b(llmi_[a-z0-9_]+)\s*\(", text)
+    # typedef'd function-pointer types are not exported symbols
+    return sorted(set(n for n in names if not n.endswith("_fn")))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = B.lib()
+    names = declared_functions()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), "libllmi_hip.so does not export " + name
+        assert name in B.SYMBOLS, "the ctypes binding does not declare " + name
+    assert set(B.SYMBOLS) == set(names)
+    assert lib.llmi_hip_abi_version() == 1
+
+
+def test_struct_layout_matches_the_c_compiler(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "llmi_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu %zu\n", sizeof(llmi_mha_args), offsetof(llmi_mha_args, layer_id),
+           offsetof(llmi_mha_args, waves_per_group), offsetof(llmi_mha_args, stream), sizeof(llmi_mha_plan));
+    printf("%zu %zu %zu %zu\n", sizeof(llmi_qk_norm_rope_args), offsetof(llmi_qk_norm_rope_args, eps),
+           offsetof(llmi_qk_norm_rope_args, stream), sizeof(llmi_pool_stats));
+    return 0;
+}
+''')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, stdout=subprocess.PIPE, text=True).stdout.split()
+    got = [int(x) for x in out]
+    want = [ctypes.sizeof(B.MhaArgs), B.MhaArgs.layer_id.offset, B.MhaArgs.waves_per_group.offset,
+            B.MhaArgs.stream.offset, ctypes.sizeof(B.MhaPlan), ctypes.sizeof(B.QkNormRopeArgs),
+            B.QkNormRopeArgs.eps.offset, B.QkNormRopeArgs.stream.offset, ctypes.sizeof(B.PoolStats)]
+    assert got == want
+
+
+def good_args(**over):
+    a = B.MhaArgs()
+    a.query = a.key_cache = a.value_cache = a.output = 0x1000
+    a.workspace = 0x2000
+    a.workspace_bytes = 64 << 20
+    a.layer_id, a.pos, a.kv_dim, a.kv_mul, a.head_num, a.head_dim, a.max_seq_len = 0, 4095, 1024, 4, 32, 128, 4096
+    for k, v in over.items():
+        setattr(a, k, v)
+    return a
+
+
+def plan(a):
+    p = B.MhaPlan()
+    rc = B.lib().llmi_hip_mha_plan(ctypes.byref(a), ctypes.byref(p))
+    return rc, p
+
+
+@pytest.mark.parametrize("over,status", [
+    (dict(query=0), "NULL_POINTER"), (dict(output=0), "NULL_POINTER"),
+    (dict(head_dim=64), "HEAD_DIM"),                      # mha_kernel.cu:478-479
+    (dict(kv_dim=1000), "KV_DIM"), (dict(kv_dim=0), "KV_DIM"),
+    (dict(head_num=31), "HEAD_GROUP"), (dict(kv_mul=0), "HEAD_GROUP"),
+    (dict(kv_mul=32, head_num=256), "HEAD_GROUP"),
+    (dict(pos=-1), "POS_RANGE"), (dict(pos=4096), "POS_RANGE"),  # mha_kernel.cu:473-474
+    (dict(query=0x1008), "ALIGNMENT"), (dict(key_cache=0x1002), "ALIGNMENT"),  # mha_kernel.cu:495-498
+    (dict(kv_layout=2), "LAYOUT"), (dict(force_path=4), "INVALID_ARG"), (dict(num_splits=257), "INVALID_ARG"),
+    (dict(waves_per_group=3), "INVALID_ARG"), (dict(layer_id=-1), "INVALID_ARG"), (dict(max_seq_len=0), "INVALID_ARG"),
+    (dict(workspace=0), "WORKSPACE"), (dict(workspace_bytes=1000), "WORKSPACE"),
+    (dict(force_path=B.PATH_SPLIT, num_splits=64, workspace_bytes=32 * 130 * 4 * 63), "WORKSPACE"),
+])
+def test_validation_status_codes(over, status):
+    rc, _ = plan(good_args(**over))
+    assert rc == B.STATUS[status], B.lib().llmi_hip_strerror(rc)
+    # the launcher validates the same way and returns before touching HIP
+    assert B.lib().llmi_hip_mha_decode(ctypes.byref(good_args(**over))) == B.STATUS[status]
+
+
+def test_null_arguments():
+    p = B.MhaPlan()
+    assert B.lib().llmi_hip_mha_plan(None, ctypes.byref(p)) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_mha_plan(ctypes.byref(good_args()), None) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_mha_decode(None) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_qk_norm_rope_append(None) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_sincos_table(None, None, 128, 16, None) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_kv_restride(None, None, 1, 16, 1024, 128, 1, None) == B.STATUS["NULL_POINTER"]
+    assert B.lib().llmi_hip_memcpy(None, None, 4, 0, None, 0) == B.STATUS["NULL_POINTER"]
+
+
+def test_plan_short_context_is_single_pass():
+    for pos in (0, 15, 16, 127, 255):
+        rc, p = plan(good_args(pos=pos, workspace=0, workspace_bytes=0))  # no workspace needed
+        assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1 and p.workspace_needed == 0
+        assert p.rows_per_split >= pos + 1 and p.rows_per_split % 16 == 0
+
+
+@pytest.mark.parametrize("ctx", [257, 1024, 4096, 8192, 32768, 131072])
+def test_plan_long_context_splits_without_empty_splits(ctx):
+    rc, p = plan(good_args(pos=ctx - 1, max_seq_len=ctx))
+    assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and 2 <= p.num_splits <= 256
+    assert p.rows_per_split % 16 == 0
+    assert (p.num_splits - 1) * p.rows_per_split < ctx <= p.num_splits * p.rows_per_split
+    assert p.workspace_needed <= B.lib().llmi_hip_mha_workspace_bytes(32, 128, ctx)
+    assert p.group_pad == 4 and p.waves_per_group in (1, 2, 4, 8)
+
+
+def test_plan_honours_requests_and_clamps_to_the_workspace():
+    rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=16))
+    assert rc == 0 and p.path == B.PATH_SPLIT and p.num_splits == 16 and p.rows_per_split == 256
+    rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=200))  # 256 tiles / 200 -> 2 tiles per split
+    assert rc == 0 and p.num_splits == 128
+    rc, p = plan(good_args(force_path=B.PATH_SINGLE_PASS))
+    assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1
+    # a reference-sized workspace [head_num, 4*max_seq_len] fp32 (qwen3_fused.cpp:502) limits the auto split count
+    small = 32 * 4 * 512 * 4
+    rc, p = plan(good_args(pos=511, max_seq_len=512, workspace_bytes=small))
+    assert rc == 0 and p.workspace_needed <= small and p.num_splits >= 2
+    # kv_mul 3 pads to 4, kv_mul 16 limits the waves per workgroup
+    rc, p = plan(good_args(kv_mul=3, head_num=24))
+    assert rc == 0 and p.group_pad == 4
+    rc, p = plan(good_args(kv_mul=16, head_num=128))
+    assert rc == 0 and p.group_pad == 16 and p.waves_per_group <= 4
+    rc, _ = plan(good_args(kv_mul=16, head_num=128, waves_per_group=8))
+    assert rc == B.STATUS["INVALID_ARG"]
+
+
+def test_workspace_bytes():
+    f = B.lib().llmi_hip_mha_workspace_bytes
+    assert f(0, 128, 100) == 0 and f(32, 128, 0) == 0
+    assert f(32, 128, 4096) >= 32 * 256 * 130 * 4
+    assert f(32, 128, 1 << 20) == f(32, 128, 4096)  # the split count is capped
+    assert f(32, 128, 64) < f(32, 128, 4096)
+
+
+def test_strerror_covers_every_status():
+    msgs = {B.lib().llmi_hip_strerror(code).decode() for code in B.STATUS.values()}
+    assert len(msgs) == len(B.STATUS) and "unknown status" not in msgs
+    assert B.lib().llmi_hip_strerror(-99).decode() == "unknown status"
+
+
+def test_qk_norm_rope_validation():
+    a = B.QkNormRopeArgs()
+    for f in ("query", "key_new", "key_cache", "norm_weight", "sin_cache", "cos_cache"):
+        setattr(a, f, 0x1000)
+    a.layer_id, a.pos, a.kv_dim, a.head_num, a.head_dim, a.max_seq_len, a.eps = 0, 5, 1024, 32, 64, 16, 1e-6
+    call = B.lib().llmi_hip_qk_norm_rope_append
+    assert call(ctypes.byref(a)) == B.STATUS["HEAD_DIM"]
+    a.head_dim = 128
+    a.pos = 16
+    assert call(ctypes.byref(a)) == B.STATUS["POS_RANGE"]
+    a.pos = 5
+    a.value_new = 0x1000  # V row given but no V cache to put it in
+    assert call(ctypes.byref(a)) == B.STATUS["NULL_POINTER"]
+    a.value_cache = 0x1000
+    a.kv_layout = 7
+    assert call(ctypes.byref(a)) == B.STATUS["LAYOUT"]
+    a.kv_layout = 0
+    a.query = 0x1001
+    assert call(ctypes.byref(a)) == B.STATUS["ALIGNMENT"]
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from llminfer_amd import _binding as B\n"
+            "B.LIB_PATH = %r\n"
+            "try:\n    B.lib()\nexcept RuntimeError as e:\n    print('RAISED', e)\n" % (ROOT, str(tmp_path / "nope.so")))
+    out = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert "RAISED" in out and "no fallback" in out
