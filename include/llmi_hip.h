@@ -118,7 +118,8 @@ int llmi_hip_mha_decode(const llmi_mha_args* args);
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len);
 
 typedef struct llmi_qk_norm_rope_args {
-    void* query;              /* device bf16 [head_num*128], normalised+rotated in place  */
+    void* query;              /* device bf16 [head_num*128]: receives the normalised+rotated query */
+    const void* query_src;    /* device bf16 [head_num*128] raw query, or NULL = transform `query` in place */
     const void* key_new;      /* device bf16 [kv_dim]: this token's K row (pre-norm)      */
     const void* value_new;    /* device bf16 [kv_dim]: this token's V row, or NULL if the
                                  V row is already in the cache                            */

@@ -43,7 +43,7 @@ class MhaPlan(ctypes.Structure):
 
 class QkNormRopeArgs(ctypes.Structure):
     _fields_ = [
-        ("query", c_void_p), ("key_new", c_void_p), ("value_new", c_void_p),
+        ("query", c_void_p), ("query_src", c_void_p), ("key_new", c_void_p), ("value_new", c_void_p),
         ("key_cache", c_void_p), ("value_cache", c_void_p), ("norm_weight", c_void_p),
         ("sin_cache", c_void_p), ("cos_cache", c_void_p),
         ("layer_id", c_i32), ("pos", c_i32), ("kv_dim", c_i32), ("head_num", c_i32),

@@ -193,7 +193,7 @@ int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {
     if (a->pos < 0 || a->pos >= a->max_seq_len) return LLMI_ERR_POS_RANGE;
     if (a->kv_layout != LLMI_KV_LAYOUT_POS_MAJOR && a->kv_layout != LLMI_KV_LAYOUT_HEAD_MAJOR)
         return LLMI_ERR_LAYOUT;
-    const void* ptrs[] = {a->query, a->key_new, a->value_new, a->key_cache, a->value_cache, a->norm_weight};
+    const void* ptrs[] = {a->query, a->query_src, a->key_new, a->value_new, a->key_cache, a->value_cache, a->norm_weight};
     for (const void* p : ptrs)
         if (p && (reinterpret_cast<uintptr_t>(p) & 3u)) return LLMI_ERR_ALIGNMENT;
     if (!(a->eps >= 0.0f)) return LLMI_ERR_INVALID_ARG;

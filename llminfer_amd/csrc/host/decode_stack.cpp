@@ -1,0 +1,139 @@
+#include "decode_stack.h"
+
+#include <hip/hip_runtime.h>
+
+#include "kernel_interface.h"
+
+namespace model {
+
+#define HIP_OK(expr)                                                                     \
+    do {                                                                                 \
+        hipError_t llmi_e_ = (expr);                                                     \
+        if (llmi_e_ != hipSuccess) LLMI_FATAL(#expr << ": " << hipGetErrorString(llmi_e_)); \
+    } while (0)
+
+DecodeStack::DecodeStack(const AttentionConfig& config) : config_(config) {
+    hip_config_ = std::make_shared<kernel::HipConfig>();
+    hip_config_->create();
+    auto alloc = base::HIPDeviceAllocatorFactory::get_instance();
+    buffers_ = std::make_unique<AttentionBuffers>(config, alloc);
+    const int32_t L = config.layer_num;
+    using base::DataType;
+    raw_q_ = tensor::Tensor(DataType::DataTypeBf16, L, config.dim(), true, alloc);
+    raw_k_ = tensor::Tensor(DataType::DataTypeBf16, L, config.kv_dim(), true, alloc);
+    raw_v_ = tensor::Tensor(DataType::DataTypeBf16, L, config.kv_dim(), true, alloc);
+    norm_w_ = tensor::Tensor(DataType::DataTypeBf16, L, 2 * config.head_dim, true, alloc);
+    outputs_ = tensor::Tensor(DataType::DataTypeBf16, L, config.dim(), true, alloc);
+    LLMI_CHECK(!raw_q_.is_empty() && !raw_k_.is_empty() && !raw_v_.is_empty() && !norm_w_.is_empty() && !outputs_.is_empty());
+}
+
+DecodeStack::~DecodeStack() {
+    if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
+    if (graph_) (void)hipGraphDestroy(graph_);
+}
+
+void DecodeStack::build_sincos() {
+    kernel::get_sin_cos_cache_kernel(base::DeviceType::DeviceHIP)(
+        buffers_->get_buffer(ModelBufferType::SinCache), buffers_->get_buffer(ModelBufferType::CosCache),
+        config_.head_dim, config_.max_seq_len, stream());
+    synchronize();
+}
+
+void DecodeStack::enqueue(int32_t pos, bool with_qk_norm_rope) {
+    const AttentionConfig& c = config_;
+    tensor::Tensor& kc = buffers_->get_buffer(ModelBufferType::KeyCache);
+    tensor::Tensor& vc = buffers_->get_buffer(ModelBufferType::ValueCache);
+    tensor::Tensor& q = buffers_->get_buffer(ModelBufferType::Query);
+    tensor::Tensor& ws = buffers_->get_buffer(ModelBufferType::KVSplitOutput);
+    for (int32_t layer = 0; layer < c.layer_num; ++layer) {
+        const void* q_for_attention = query_raw(layer);
+        if (with_qk_norm_rope) {
+            llmi_qk_norm_rope_args a{};
+            a.query = q.ptr<uint16_t>();
+            a.query_src = query_raw(layer);
+            a.key_new = key_raw(layer);
+            a.value_new = value_raw(layer);
+            a.key_cache = kc.ptr<uint16_t>();
+            a.value_cache = vc.ptr<uint16_t>();
+            a.norm_weight = norm_weight(layer);
+            a.sin_cache = buffers_->get_buffer(ModelBufferType::SinCache).ptr<float>();
+            a.cos_cache = buffers_->get_buffer(ModelBufferType::CosCache).ptr<float>();
+            a.layer_id = layer;
+            a.pos = pos;
+            a.kv_dim = c.kv_dim();
+            a.head_num = c.head_num;
+            a.head_dim = c.head_dim;
+            a.max_seq_len = c.max_seq_len;
+            a.kv_layout = c.kv_layout;
+            a.eps = 1e-6f;
+            a.stream = stream();
+            const int rc = llmi_hip_qk_norm_rope_append(&a);
+            if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_qk_norm_rope_append: " << llmi_hip_strerror(rc));
+            q_for_attention = q.ptr<uint16_t>();
+        }
+        llmi_mha_args m{};
+        m.query = q_for_attention;
+        m.key_cache = kc.ptr<uint16_t>();
+        m.value_cache = vc.ptr<uint16_t>();
+        m.workspace = ws.ptr<float>();
+        m.workspace_bytes = ws.byte_size();
+        m.output = output(layer);
+        m.layer_id = layer;
+        m.pos = pos;
+        m.kv_dim = c.kv_dim();
+        m.kv_mul = c.kv_mul();
+        m.head_num = c.head_num;
+        m.head_dim = c.head_dim;
+        m.max_seq_len = c.max_seq_len;
+        m.kv_layout = c.kv_layout;
+        const kernel::MhaHipOptions& o = kernel::mha_hip_options();
+        m.force_path = o.force_path;
+        m.num_splits = o.num_splits;
+        m.waves_per_group = o.waves_per_group;
+        m.stream = stream();
+        const int rc = llmi_hip_mha_decode(&m);
+        if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_mha_decode: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
+    }
+}
+
+void DecodeStack::capture(int32_t pos, bool with_qk_norm_rope) {
+    if (graph_exec_) {
+        HIP_OK(hipGraphExecDestroy(graph_exec_));
+        graph_exec_ = nullptr;
+    }
+    if (graph_) {
+        HIP_OK(hipGraphDestroy(graph_));
+        graph_ = nullptr;
+    }
+    HIP_OK(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
+    try {
+        enqueue(pos, with_qk_norm_rope);
+    } catch (...) {
+        hipGraph_t dead = nullptr;
+        (void)hipStreamEndCapture(stream(), &dead);
+        if (dead) (void)hipGraphDestroy(dead);
+        throw;
+    }
+    HIP_OK(hipStreamEndCapture(stream(), &graph_));
+    HIP_OK(hipGraphInstantiate(&graph_exec_, graph_, nullptr, nullptr, 0));
+}
+
+float DecodeStack::replay(int32_t times) {
+    LLMI_CHECK(graph_exec_ != nullptr);
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    HIP_OK(hipEventRecord(e0, stream()));
+    for (int32_t i = 0; i < times; ++i) HIP_OK(hipGraphLaunch(graph_exec_, stream()));
+    HIP_OK(hipEventRecord(e1, stream()));
+    HIP_OK(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    HIP_OK(hipEventDestroy(e0));
+    HIP_OK(hipEventDestroy(e1));
+    return ms;
+}
+
+void DecodeStack::synchronize() { HIP_OK(hipStreamSynchronize(stream())); }
+
+}  // namespace model

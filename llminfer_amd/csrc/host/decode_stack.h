@@ -1,0 +1,54 @@
+// The attention part of one decode step over all layers, as the engine's layer
+// loop issues it (code/source/model/qwen3_fused.cpp:115-127 with :517-553):
+// per layer, fused QK-Norm + RoPE on the new token's Q and K with the K and V
+// rows appended to the cache, then grouped-query attention over positions
+// 0..pos. The sequence can be captured once into a HIP graph and replayed.
+// Harness for benchmarks and tests, not part of the C ABI.
+#ifndef LLMI_HOST_DECODE_STACK_H
+#define LLMI_HOST_DECODE_STACK_H
+
+#include <memory>
+#include <vector>
+
+#include "attention_buffers.h"
+#include "hip_config.h"
+
+namespace model {
+
+class DecodeStack {
+public:
+    explicit DecodeStack(const AttentionConfig& config);
+    ~DecodeStack();
+    DecodeStack(const DecodeStack&) = delete;
+    DecodeStack& operator=(const DecodeStack&) = delete;
+
+    AttentionBuffers& buffers() { return *buffers_; }
+    hipStream_t stream() const { return hip_config_->stream; }
+    // Per-layer inputs of the new token (raw, before QK-Norm) and norm weights, device bf16.
+    uint16_t* query_raw(int32_t layer) { return raw_q_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.dim()); }
+    uint16_t* key_raw(int32_t layer) { return raw_k_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.kv_dim()); }
+    uint16_t* value_raw(int32_t layer) { return raw_v_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.kv_dim()); }
+    uint16_t* norm_weight(int32_t layer) { return norm_w_.ptr<uint16_t>(static_cast<int64_t>(layer) * 2 * config_.head_dim); }
+    // Per-layer attention outputs [layer][dim], device bf16.
+    uint16_t* output(int32_t layer) { return outputs_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.dim()); }
+
+    void build_sincos();
+    // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
+    void enqueue(int32_t pos, bool with_qk_norm_rope);
+    // Captures enqueue(pos) into a graph (replacing an earlier one).
+    void capture(int32_t pos, bool with_qk_norm_rope);
+    // Replays the captured graph `times` times; returns the elapsed milliseconds (HIP events on the stream).
+    float replay(int32_t times);
+    void synchronize();
+
+private:
+    AttentionConfig config_;
+    std::shared_ptr<kernel::HipConfig> hip_config_;
+    std::unique_ptr<AttentionBuffers> buffers_;
+    tensor::Tensor raw_q_, raw_k_, raw_v_, norm_w_, outputs_;
+    hipGraph_t graph_ = nullptr;
+    hipGraphExec_t graph_exec_ = nullptr;
+};
+
+}  // namespace model
+#endif

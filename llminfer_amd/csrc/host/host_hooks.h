@@ -1,0 +1,41 @@
+// C entry points into the C++ host layer for drivers that are not C++ (the
+// Python benchmark and tests, through ctypes). A harness interface: the
+// drop-in boundary is include/llmi_hip.h.
+#ifndef LLMI_HOST_HOOKS_H
+#define LLMI_HOST_HOOKS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct llmi_host_stack llmi_host_stack;
+
+/* Last error message of a failed hook on this thread ("" if none). Hooks return 0 / non-NULL on success. */
+const char* llmi_host_last_error(void);
+
+llmi_host_stack* llmi_host_stack_create(int32_t layer_num, int32_t max_seq_len, int32_t head_num,
+                                        int32_t kv_head_num, int32_t kv_layout);
+void llmi_host_stack_destroy(llmi_host_stack* s);
+/* which: 0 key cache base, 1 value cache base, 2 raw query of `layer`, 3 raw key, 4 raw value,
+ * 5 norm weight, 6 output of `layer`, 7 sin table, 8 cos table, 9 normalised query buffer. Device pointers. */
+void* llmi_host_stack_ptr(llmi_host_stack* s, int32_t which, int32_t layer);
+int llmi_host_stack_build_sincos(llmi_host_stack* s);
+int llmi_host_stack_run(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);      /* eager + synchronise */
+int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);
+int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms);
+/* Process-wide tuning overrides of the HIP attention arm (0 = automatic). */
+void llmi_host_set_mha_options(int32_t force_path, int32_t num_splits, int32_t waves_per_group);
+
+/* Runs op::MultiHeadAttention::forward through the registry on borrowed device pointers; returns the
+ * base::Status code (0 = success), -1 for a fatal error. cache_dims is 3 (position-major) or 4 (head-major). */
+int llmi_host_mha_forward(void* query, void* key_cache, void* value_cache, void* workspace, int64_t workspace_floats,
+                          void* output, int32_t layer_num, int32_t layer_id, int32_t pos, int32_t kv_dim,
+                          int32_t kv_mul, int32_t head_num, int32_t head_dim, int32_t max_seq_len,
+                          int32_t cache_dims);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

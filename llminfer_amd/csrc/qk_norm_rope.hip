@@ -32,6 +32,7 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
 
 struct AppendArgs {
     uint16_t* query;
+    const uint16_t* query_src;
     const uint16_t* key_new;
     const uint16_t* value_new;
     uint16_t* key_slot;    // cache address of (layer, pos, kv_head 0)
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(kHalf) void qk_norm_rope_append_kernel(AppendArgs a
     uint16_t* dst;
     const uint16_t* w;
     if (b < a.head_num) {
-        src = a.query + b * kHeadDim;
+        src = a.query_src + b * kHeadDim;
         dst = a.query + b * kHeadDim;
         w = a.weight;
     } else {
@@ -131,6 +132,7 @@ int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args) {
     }
     AppendArgs a;
     a.query = static_cast<uint16_t*>(args.query);
+    a.query_src = args.query_src ? static_cast<const uint16_t*>(args.query_src) : a.query;
     a.key_new = static_cast<const uint16_t*>(args.key_new);
     a.value_new = static_cast<const uint16_t*>(args.value_new);
     a.key_slot = static_cast<uint16_t*>(args.key_cache) + slot_off;

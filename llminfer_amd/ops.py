@@ -88,14 +88,14 @@ def mha_decode_raw(args):
 
 def qk_norm_rope_append(query, key_new, value_new, key_cache, value_cache, norm_weight, sin_cache, cos_cache, *,
                         layer_id, pos, kv_dim, head_num, head_dim, max_seq_len,
-                        kv_layout=B.KV_LAYOUT_POS_MAJOR, eps=1e-6, stream=None):
-    for name, t in (("query", query), ("key_new", key_new), ("value_new", value_new),
+                        kv_layout=B.KV_LAYOUT_POS_MAJOR, eps=1e-6, query_src=None, stream=None):
+    for name, t in (("query", query), ("query_src", query_src), ("key_new", key_new), ("value_new", value_new),
                     ("key_cache", key_cache), ("value_cache", value_cache), ("norm_weight", norm_weight)):
         _check_dev(name, t, _BF16_DTYPES)
     _check_dev("sin_cache", sin_cache, (torch.float32,))
     _check_dev("cos_cache", cos_cache, (torch.float32,))
     a = B.QkNormRopeArgs()
-    a.query, a.key_new, a.value_new = _ptr(query), _ptr(key_new), _ptr(value_new)
+    a.query, a.query_src, a.key_new, a.value_new = _ptr(query), _ptr(query_src), _ptr(key_new), _ptr(value_new)
     a.key_cache, a.value_cache, a.norm_weight = _ptr(key_cache), _ptr(value_cache), _ptr(norm_weight)
     a.sin_cache, a.cos_cache = _ptr(sin_cache), _ptr(cos_cache)
     a.layer_id, a.pos, a.kv_dim, a.head_num = layer_id, pos, kv_dim, head_num

@@ -1,0 +1,275 @@
+"""GPU tests of the per-token writers (fused QK-Norm + RoPE + K/V append, sin/cos table, cache re-stride),
+of the pooled device allocator, and of the captured multi-layer decode stack, against the CPU oracle."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from llminfer_amd import _binding as B
+from llminfer_amd import ops, synth
+
+from helpers import assert_parity, from_dev_bf16, to_dev
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _bf16_close(got_bits, want_bits, what):
+    """Outputs of the fused norm/rope chain: at most one bf16 ulp apart, and almost all identical. The
+    reference's own tolerance for this op is atol = rtol = 2e-2 (test_qwen3_bf16_ops.py:836-917)."""
+    g = synth.bf16_bits_to_f32(got_bits).astype(np.float64)
+    w = synth.bf16_bits_to_f32(want_bits).astype(np.float64)
+    assert np.all(np.abs(g - w) <= np.abs(w) / 128 + 1e-6), what
+    assert (got_bits == want_bits).mean() > 0.99, what
+
+
+def test_sincos_table_matches_oracle(oracle, dev):
+    sin_d, cos_d = ops.sincos_table(128, 5000, dev)
+    torch.cuda.synchronize()
+    sin_o, cos_o = oracle.sincos_table(128, 5000)
+    # the reference's own tolerance for this table is 2e-6 (test_qwen3_bf16_ops.py:857-858)
+    assert np.abs(sin_d.cpu().numpy() - sin_o).max() <= 2e-6
+    assert np.abs(cos_d.cpu().numpy() - cos_o).max() <= 2e-6
+
+
+@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
+@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (64, 8), (16, 8)])
+def test_qk_norm_rope_append(oracle, dev, layout, n_q, n_kv):
+    rng = np.random.RandomState(n_q + layout)
+    d, layers, msl, layer_id, pos = 128, 3, 50, 2, 41
+    kv_dim = n_kv * d
+    q = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+    k_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    v_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+    sin_o, cos_o = oracle.sincos_table(d, msl)
+    q_ref = oracle.qk_norm_rope(q, w[:d], sin_o[pos], cos_o[pos])
+    k_ref = oracle.qk_norm_rope(k_new, w[d:], sin_o[pos], cos_o[pos])
+
+    cache_shape = (layers, msl, kv_dim) if layout == 0 else (layers, n_kv, msl, d)
+    k_cache = torch.full(cache_shape, 0x1234, dtype=torch.int16, device=dev)
+    v_cache = torch.full(cache_shape, 0x1234, dtype=torch.int16, device=dev)
+    q_d = torch.zeros(n_q * d, dtype=torch.int16, device=dev)
+    sin_d, cos_d = ops.sincos_table(d, msl, dev)
+    ops.qk_norm_rope_append(q_d, to_dev(k_new.reshape(-1), dev), to_dev(v_new.reshape(-1), dev), k_cache, v_cache,
+                            to_dev(w, dev), sin_d, cos_d, layer_id=layer_id, pos=pos, kv_dim=kv_dim, head_num=n_q,
+                            head_dim=d, max_seq_len=msl, kv_layout=layout, query_src=to_dev(q.reshape(-1), dev))
+    torch.cuda.synchronize()
+    _bf16_close(q_d.cpu().numpy().view(np.uint16).reshape(n_q, d), q_ref, "query")
+    kc = k_cache.cpu().numpy().view(np.uint16)
+    vc = v_cache.cpu().numpy().view(np.uint16)
+    if layout == 0:
+        k_row, v_row = kc[layer_id, pos].reshape(n_kv, d), vc[layer_id, pos].reshape(n_kv, d)
+        kc[layer_id, pos] = 0x1234
+        vc[layer_id, pos] = 0x1234
+    else:
+        k_row, v_row = kc[layer_id, :, pos].copy(), vc[layer_id, :, pos].copy()
+        kc[layer_id, :, pos] = 0x1234
+        vc[layer_id, :, pos] = 0x1234
+    _bf16_close(k_row, k_ref, "key row")
+    assert np.array_equal(v_row, v_new)                    # V is copied bit for bit
+    assert np.all(kc == 0x1234) and np.all(vc == 0x1234)  # nothing else in the caches was touched
+
+
+def test_qk_norm_rope_in_place_on_the_cache_row(oracle, dev):
+    """The reference's call pattern: K row already in its position-major cache slot, transformed in place,
+    V untouched (rmsnorm_kernel.cu:248-290 with model.cpp:90-107)."""
+    rng = np.random.RandomState(3)
+    d, n_q, n_kv, msl, pos = 128, 32, 8, 16, 9
+    q = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+    cache = synth.f32_to_bf16_bits(rng.standard_normal((1, msl, n_kv * d)).astype(np.float32))
+    w = synth.f32_to_bf16_bits(np.ones(2 * d, dtype=np.float32))
+    sin_o, cos_o = oracle.sincos_table(d, msl)
+    k_ref = oracle.qk_norm_rope(cache[0, pos].reshape(n_kv, d), w[d:], sin_o[pos], cos_o[pos])
+    q_ref = oracle.qk_norm_rope(q, w[:d], sin_o[pos], cos_o[pos])
+    k_cache = to_dev(cache, dev)
+    q_d = to_dev(q.reshape(-1), dev)
+    sin_d, cos_d = ops.sincos_table(d, msl, dev)
+    row = k_cache[0, pos]  # contiguous view of the slot
+    ops.qk_norm_rope_append(q_d, row, None, k_cache, None, to_dev(w, dev), sin_d, cos_d, layer_id=0, pos=pos,
+                            kv_dim=n_kv * d, head_num=n_q, head_dim=d, max_seq_len=msl)
+    torch.cuda.synchronize()
+    got = k_cache.cpu().numpy().view(np.uint16)
+    _bf16_close(got[0, pos].reshape(n_kv, d), k_ref, "key row")
+    _bf16_close(q_d.cpu().numpy().view(np.uint16).reshape(n_q, d), q_ref, "query")
+    mask = np.ones(msl, dtype=bool)
+    mask[pos] = False
+    assert np.array_equal(got[0, mask], cache[0, mask])
+
+
+def test_kv_restride_is_a_permutation(dev):
+    layers, msl, n_kv, d, num_pos = 3, 37, 8, 128, 30
+    src = np.random.RandomState(0).randint(0, 65536, size=(layers, msl, n_kv * d)).astype(np.uint16)
+    dst = torch.zeros((layers, n_kv, msl, d), dtype=torch.int16, device=dev)
+    ops.kv_restride(to_dev(src, dev), dst, layer_num=layers, max_seq_len=msl, kv_dim=n_kv * d, head_dim=d,
+                    num_pos=num_pos)
+    torch.cuda.synchronize()
+    got = dst.cpu().numpy().view(np.uint16)
+    want = synth.to_head_major(src, n_kv)
+    assert np.array_equal(got[:, :, :num_pos], want[:, :, :num_pos])
+    assert not got[:, :, num_pos:].any()  # rows past num_pos are left alone
+
+
+def test_attention_after_append_uses_the_new_row(oracle, dev):
+    """Append token `pos` with the fused kernel, then attend over 0..pos: equals the oracle run on a cache
+    whose row `pos` holds the oracle's normalised K row and the raw V row."""
+    rng = np.random.RandomState(8)
+    n_q, n_kv, d, ctx = 32, 8, 128, 600
+    case = synth.make_case(55, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=ctx + 1)
+    pos = ctx
+    q_raw = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+    k_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    v_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+    sin_o, cos_o = oracle.sincos_table(d, ctx + 1)
+    q_n = oracle.qk_norm_rope(q_raw, w[:d], sin_o[pos], cos_o[pos])
+    k_ref, v_ref = case["k"].copy(), case["v"].copy()
+    k_ref[0, pos] = oracle.qk_norm_rope(k_new, w[d:], sin_o[pos], cos_o[pos]).reshape(-1)
+    v_ref[0, pos] = v_new.reshape(-1)
+    ref = oracle.mha_cpu(q_n.reshape(-1), k_ref, v_ref, 0, pos, n_kv * d, n_q // n_kv, n_q, d, ctx + 1)
+
+    k_d = to_dev(synth.to_head_major(case["k"], n_kv), dev)
+    v_d = to_dev(synth.to_head_major(case["v"], n_kv), dev)
+    q_d = torch.zeros(n_q * d, dtype=torch.int16, device=dev)
+    out = torch.zeros(n_q * d, dtype=torch.int16, device=dev)
+    ws = torch.empty(ops.workspace_bytes(n_q, d, ctx + 1) // 4, dtype=torch.float32, device=dev)
+    sin_d, cos_d = ops.sincos_table(d, ctx + 1, dev)
+    kw = dict(layer_id=0, pos=pos, kv_dim=n_kv * d, head_num=n_q, head_dim=d, max_seq_len=ctx + 1,
+              kv_layout=B.KV_LAYOUT_HEAD_MAJOR)
+    ops.qk_norm_rope_append(q_d, to_dev(k_new.reshape(-1), dev), to_dev(v_new.reshape(-1), dev), k_d, v_d,
+                            to_dev(w, dev), sin_d, cos_d, query_src=to_dev(q_raw.reshape(-1), dev), **kw)
+    ops.mha_decode(q_d, k_d, v_d, out, ws, kv_mul=n_q // n_kv, **kw)
+    torch.cuda.synchronize()
+    assert_parity(from_dev_bf16(out), ref, "append + attention")
+
+
+def test_default_pool_on_device(dev):
+    lib = B.lib()
+    a = lib.llmi_hip_pool_alloc(4)
+    assert a and lib.llmi_hip_pool_free(a) == 0
+    assert lib.llmi_hip_pool_alloc(4) == a
+    big = lib.llmi_hip_pool_alloc(5 << 20)
+    assert big and lib.llmi_hip_memset_zero(big, 5 << 20, None, 1) == 0
+    host = (ctypes.c_uint8 * 16)(*range(16))
+    back = (ctypes.c_uint8 * 16)()
+    assert lib.llmi_hip_memcpy(big, host, 16, 1, None, 1) == 0
+    assert lib.llmi_hip_memcpy(back, big, 16, 2, None, 1) == 0
+    assert list(back) == list(range(16))
+    assert lib.llmi_hip_pool_free(big) == 0 and lib.llmi_hip_pool_free(big) == B.STATUS["UNKNOWN_POINTER"]
+    assert lib.llmi_hip_pool_alloc((5 << 20) - 4096) == big
+
+
+# ---------------------------------------------------------------- the captured multi-layer stack
+class HostLib:
+    def __init__(self):
+        L = ctypes.CDLL(os.path.join(ROOT, "llminfer_amd", "libllmi_host.so"))
+        L.llmi_host_stack_create.restype = ctypes.c_void_p
+        L.llmi_host_stack_create.argtypes = [ctypes.c_int32] * 5
+        L.llmi_host_stack_destroy.argtypes = [ctypes.c_void_p]
+        L.llmi_host_stack_ptr.restype = ctypes.c_void_p
+        L.llmi_host_stack_ptr.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+        for name in ("llmi_host_stack_build_sincos",):
+            getattr(L, name).argtypes = [ctypes.c_void_p]
+        L.llmi_host_stack_run.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+        L.llmi_host_stack_capture.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+        L.llmi_host_stack_replay.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_float)]
+        L.llmi_host_last_error.restype = ctypes.c_char_p
+        L.llmi_host_mha_forward.argtypes = ([ctypes.c_void_p] * 4 + [ctypes.c_int64, ctypes.c_void_p] +
+                                            [ctypes.c_int32] * 9)
+        self.L = L
+
+    def ok(self, rc):
+        assert rc == 0, self.L.llmi_host_last_error().decode()
+
+
+def _upload(ptr, arr):
+    arr = np.ascontiguousarray(arr)
+    rc = B.lib().llmi_hip_memcpy(ptr, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes, 1, None, 1)
+    assert rc == 0
+
+
+def _download(ptr, shape, dtype):
+    out = np.empty(shape, dtype=dtype)
+    assert B.lib().llmi_hip_memcpy(out.ctypes.data_as(ctypes.c_void_p), ptr, out.nbytes, 2, None, 1) == 0
+    return out
+
+
+@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
+def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout):
+    """4 layers of (QK-Norm + RoPE + append, attention) at ctx 300 + 1 new token: eager run and several
+    replays of the captured graph all match the oracle layer by layer."""
+    H = HostLib()
+    layers, ctx, n_q, n_kv, d = 4, 300, 32, 8, 128
+    msl, pos, kv_dim = ctx + 1, ctx, n_kv * d
+    stack = H.L.llmi_host_stack_create(layers, msl, n_q, n_kv, layout)
+    assert stack, H.L.llmi_host_last_error().decode()
+    try:
+        H.ok(H.L.llmi_host_stack_build_sincos(stack))
+        rng = np.random.RandomState(4)
+        k_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        v_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        raw = []
+        for l in range(layers):
+            c = synth.make_case(400 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+            k_all[l], v_all[l] = c["k"][0], c["v"][0]
+            qr = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+            kr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+            vr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+            w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+            raw.append((qr, kr, vr, w))
+            for which, arr in ((2, qr), (3, kr), (4, vr), (5, w)):
+                _upload(H.L.llmi_host_stack_ptr(stack, which, l), arr)
+        k_up = k_all if layout == 0 else synth.to_head_major(k_all, n_kv)
+        v_up = v_all if layout == 0 else synth.to_head_major(v_all, n_kv)
+        _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up)
+        _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), v_up)
+
+        sin_o, cos_o = oracle.sincos_table(d, msl)
+        refs = []
+        for l in range(layers):
+            qr, kr, vr, w = raw[l]
+            k_ref, v_ref = k_all[l:l + 1].copy(), v_all[l:l + 1].copy()
+            k_ref[0, pos] = oracle.qk_norm_rope(kr, w[d:], sin_o[pos], cos_o[pos]).reshape(-1)
+            v_ref[0, pos] = vr.reshape(-1)
+            qn = oracle.qk_norm_rope(qr, w[:d], sin_o[pos], cos_o[pos]).reshape(-1)
+            refs.append(oracle.mha_cpu(qn, k_ref, v_ref, 0, pos, kv_dim, n_q // n_kv, n_q, d, msl))
+
+        def check(tag):
+            for l in range(layers):
+                got = _download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16)
+                assert_parity(synth.bf16_bits_to_f32(got), refs[l], "%s layer %d" % (tag, l))
+
+        H.ok(H.L.llmi_host_stack_run(stack, pos, 1))
+        check("eager")
+        H.ok(H.L.llmi_host_stack_capture(stack, pos, 1))
+        ms = ctypes.c_float()
+        for rep in range(3):
+            for l in range(layers):  # wipe the outputs between replays
+                _upload(H.L.llmi_host_stack_ptr(stack, 6, l), np.zeros(n_q * d, dtype=np.uint16))
+            H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
+            check("replay %d" % rep)
+            torch.randn(1000, device=dev).sum().item()  # eager work between replays
+        assert ms.value > 0
+    finally:
+        H.L.llmi_host_stack_destroy(stack)
+
+
+def test_mha_op_forward_through_registry_hook(oracle, dev):
+    """op::MultiHeadAttention::forward (C++ op layer -> registry -> HIP arm) on borrowed device tensors."""
+    H = HostLib()
+    case = synth.make_case(61, n_q=32, n_kv=8, ctx=1111, max_seq_len=1200, layers=2, layer_id=1)
+    ref = oracle.mha_cpu(case["q"], case["k"], case["v"], 1, 1110, 1024, 4, 32, 128, 1200)
+    q, k, v = to_dev(case["q"], dev), to_dev(case["k"], dev), to_dev(case["v"], dev)
+    out = torch.zeros(32 * 128, dtype=torch.int16, device=dev)
+    ws = torch.empty(32 * 4 * 1200, dtype=torch.float32, device=dev)  # the reference's [head_num, 4*max_seq_len]
+    rc = H.L.llmi_host_mha_forward(q.data_ptr(), k.data_ptr(), v.data_ptr(), ws.data_ptr(), ws.numel(),
+                                   out.data_ptr(), 2, 1, 1110, 1024, 4, 32, 128, 1200, 3)
+    assert rc == 0, H.L.llmi_host_last_error().decode()
+    assert_parity(from_dev_bf16(out), ref, "op layer forward")
+    # a workspace smaller than the op's check() accepts is an InvalidArgument status (7), not a launch
+    rc = H.L.llmi_host_mha_forward(q.data_ptr(), k.data_ptr(), v.data_ptr(), ws.data_ptr(), 32 * 100,
+                                   out.data_ptr(), 2, 1, 1110, 1024, 4, 32, 128, 1200, 3)
+    assert rc == 7

@@ -174,7 +174,7 @@ def test_qk_norm_rope_validation():
     a.kv_layout = 7
     assert call(ctypes.byref(a)) == B.STATUS["LAYOUT"]
     a.kv_layout = 0
-    a.query = 0x1001
+    a.query_src = 0x1001
     assert call(ctypes.byref(a)) == B.STATUS["ALIGNMENT"]
 
 
