@@ -62,7 +62,7 @@ def test_qk_norm_rope_append(oracle, dev, layout, n_q, n_kv):
     kc = k_cache.cpu().numpy().view(np.uint16)
     vc = v_cache.cpu().numpy().view(np.uint16)
     if layout == 0:
-        k_row, v_row = kc[layer_id, pos].reshape(n_kv, d), vc[layer_id, pos].reshape(n_kv, d)
+        k_row, v_row = kc[layer_id, pos].reshape(n_kv, d).copy(), vc[layer_id, pos].reshape(n_kv, d).copy()
         kc[layer_id, pos] = 0x1234
         vc[layer_id, pos] = 0x1234
     else:
