@@ -96,7 +96,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
     if (max_waves > kMaxWaves) max_waves = kMaxWaves;
     if (a->waves_per_group > max_waves) return LLMI_ERR_INVALID_ARG;
     const size_t per_split_plain = (size_t)a->head_num * (a->head_dim + 2) * sizeof(float);
-    const size_t per_split_fused = per_split_plain + (size_t)n_kv * sizeof(unsigned long long);
+    // fused combine: per head and split, 128 partial outputs and two 8-byte arrival records
+    const size_t per_split_fused = (size_t)a->head_num * (a->head_dim * sizeof(float) + 2 * sizeof(unsigned long long));
 
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
@@ -108,7 +109,6 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
 
     int num_splits = 1, tiles_per_split = tiles, waves;
     if (path != LLMI_PATH_SINGLE_PASS) {
-        // The fused combine keeps one 8-byte arrival flag per (KV head, split) behind the partials.
         const bool fused = path == LLMI_PATH_SPLIT_FUSED;
         waves = a->waves_per_group ? a->waves_per_group : (max_waves < 4 ? max_waves : 4);
         int want = a->num_splits;
@@ -177,9 +177,9 @@ size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t 
     if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     int splits = (max_seq_len + kTile - 1) / kTile;
     if (splits > kMaxSplits) splits = kMaxSplits;
-    // Partials for the largest split count plus the arrival flags of the fused combine
-    // (one per KV head and split; head_num bounds the KV head count).
-    return (size_t)head_num * (size_t)splits * ((size_t)(head_dim + 2) * sizeof(float) + sizeof(unsigned long long)) + 16;
+    // Per head and split: head_dim partial outputs plus either (max, sum) as two floats
+    // (separate combine kernel) or two 8-byte arrival records (fused combine).
+    return (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16;
 }
 
 int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {

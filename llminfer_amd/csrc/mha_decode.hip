@@ -93,12 +93,21 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // lane L's bytes land at lds_off + 16*L. `base` and `lds_off` are wave-uniform,
 // `voff` is the lane's byte offset from base. Counted by vmcnt like any load.
 __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t lds_off) {
+    // The instruction takes its base and the LDS offset (through M0) from scalar
+    // registers; readfirstlane guarantees that whatever the surrounding code
+    // made of these wave-uniform values (it is free when they already are scalar).
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    // (the builtin returns a signed int: go through uint32_t so that the low half is not sign-extended)
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    const uint64_t sbase = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    const uint32_t slds = (uint32_t)__builtin_amdgcn_readfirstlane(lds_off);
 #if LLMI_NT_LOADS
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
-                 :: "s"(lds_off), "v"(voff), "s"(base) : "memory");
+                 :: "s"(slds), "v"(voff), "s"(sbase) : "memory");
 #else
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_off), "v"(voff), "s"(base) : "memory");
+                 :: "s"(slds), "v"(voff), "s"(sbase) : "memory");
 #endif
 }
 
@@ -122,7 +131,7 @@ struct KernelArgs {
     float* ws;            // split partials (num_splits > 1)
     uint16_t* out;        // [n_kv*group][128]
     float* out_f32;       // optional
-    unsigned long long* arrivals;  // [n_kv][num_splits] arrival flags of the fused combine, or nullptr
+    unsigned long long* records;   // [n_q][num_splits][2] arrival records of the fused combine, or nullptr
     unsigned long long epoch;      // tag of this call, 48 bits
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
@@ -189,8 +198,12 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // tile read the last valid row and are masked out of the softmax.
     constexpr int kStageBytes = 8192;
     constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
-    constexpr int kMergeBytes = NW * G * (kHeadDim + 2) * (int)sizeof(float);
-    constexpr int kCombineBytes = (G * kMaxSplits + G) * (int)sizeof(float);
+    // Merge area: NW x kRows x G x 128 partial outputs + per-wave and merged (max, sum) pairs.
+    constexpr int kMergeTail = (2 * NW * G + 2 * G) * (int)sizeof(float);
+    constexpr int kMerge4 = NW * 4 * G * kHeadDim * (int)sizeof(float) + kMergeTail;
+    constexpr int kRows = kMerge4 <= 65536 ? 4 : 1;
+    constexpr int kMergeBytes = NW * kRows * G * kHeadDim * (int)sizeof(float) + kMergeTail;
+    constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float);
     constexpr int kSmemBytes = kRingBytes > kMergeBytes ? (kRingBytes > kCombineBytes ? kRingBytes : kCombineBytes)
                                                         : (kMergeBytes > kCombineBytes ? kMergeBytes : kCombineBytes);
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
@@ -287,41 +300,49 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
     }
 
-    // Fold the four DPP rows of the wave together (same head / same columns).
+    // ---- epilogue: fold the wave's four DPP rows and the workgroup's waves ----
+    // Each DPP row (kg) holds a partial sum over its own positions; all rows share
+    // the running max of a head, so rows add up plainly. When LDS has room the
+    // four rows are written side by side and summed by the merge below (no
+    // cross-lane traffic at all); otherwise they are folded with xor shuffles first.
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
+    if constexpr (kRows == 1) {
 #pragma unroll
-    for (int h = 0; h < G; ++h)
+        for (int h = 0; h < G; ++h)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float x = o[h][e];
-            x += __shfl_xor(x, 16);
-            x += __shfl_xor(x, 32);
-            o[h][e] = x;
-        }
+            for (int e = 0; e < 8; ++e) {
+                float x = o[h][e];
+                x += __shfl_xor(x, 16);
+                x += __shfl_xor(x, 32);
+                o[h][e] = x;
+            }
+    }
 
-    // Merge the waves of the workgroup through LDS (the ring is drained: every
-    // tile issued was waited for; reuse its memory once all waves are done with it).
+    // The ring is drained (every tile issued was waited for): reuse its memory
+    // once all waves are done with it.
     __syncthreads();
-    typedef float (*MergeO)[G][kHeadDim];
+    typedef float (*MergeO)[kRows][G][kHeadDim];
     typedef float (*MergeS)[G];
     MergeO s_o = reinterpret_cast<MergeO>(smem);
-    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * G * kHeadDim * sizeof(float));
-    MergeS s_l = reinterpret_cast<MergeS>(smem + NW * G * (kHeadDim + 1) * sizeof(float));
-    if (kg == 0) {
+    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * kRows * G * kHeadDim * sizeof(float));
+    MergeS s_l = s_m + NW;
+    float* s_fin = reinterpret_cast<float*>(s_l + NW);  // [G][2]: merged (max, sum) per head
+    if (kRows == 4 || kg == 0) {
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-            float* dst = &s_o[wave][h][n16 * 8];
+            float* dst = &s_o[wave][kRows == 4 ? kg : 0][h][n16 * 8];
             *reinterpret_cast<f32x4*>(dst) = f32x4{o[h][0], o[h][1], o[h][2], o[h][3]};
             *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[h][4], o[h][5], o[h][6], o[h][7]};
         }
-        if (n16 < G) {
-            s_m[wave][n16] = m_run;
-            s_l[wave][n16] = l_run;
-        }
+    }
+    if (kg == 0 && n16 < G) {
+        s_m[wave][n16] = m_run;
+        s_l[wave][n16] = l_run;
     }
     __syncthreads();
 
+    const bool fused = a.records != nullptr && a.num_splits > 1;
     const int n_out = a.group * kHeadDim;
     for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
         const int h = idx >> 7;
@@ -334,7 +355,10 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         for (int w = 0; w < NW; ++w) {
             const float mw = s_m[w][h];
             const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - mx);
-            acc += s_o[w][h][d] * f;
+            float rows = s_o[w][0][h][d];
+#pragma unroll
+            for (int r = 1; r < kRows; ++r) rows += s_o[w][r][h][d];
+            acc += rows * f;
             lsum += s_l[w][h] * f;
         }
         const int hq = kvh * a.group + h;
@@ -345,90 +369,113 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         } else {
             const int64_t S = a.num_splits;
             float* po = a.ws + ((int64_t)hq * S + split) * kHeadDim + d;
-            float* pm = a.ws + (int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split;
-            float* pl = a.ws + (int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split;
-            if (a.arrivals) {
-                // Device-coherent stores: they go past this XCD's L2, so the
-                // workgroup (possibly on another XCD) that does the combine can
-                // read them without anyone flushing or invalidating a cache.
+            if (fused) {
+                // Device-coherent store: it goes past this XCD's L2, so the workgroup
+                // (possibly on another XCD) that does the combine can read it without
+                // anyone flushing or invalidating a cache.
                 __hip_atomic_store(po, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (d == 0) {
-                    __hip_atomic_store(pm, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(pl, lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_fin[2 * h] = mx;
+                    s_fin[2 * h + 1] = lsum;
                 }
             } else {
                 *po = acc;
                 if (d == 0) {
-                    *pm = mx;
-                    *pl = lsum;
+                    a.ws[(int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split] = mx;
+                    a.ws[(int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split] = lsum;
                 }
             }
         }
     }
+    if (!fused) return;
 
-    // Fused combine: the workgroup of the LAST split of this KV head merges the
-    // partials of its query heads, so no second launch is needed. Every split
-    // publishes a flag after its partials; the last split's workgroup waits for
-    // all flags. Workgroups are dispatched in index order and the others never
-    // wait for anything, so whoever it waits for is already running or done.
-    if (a.num_splits == 1 || a.arrivals == nullptr) return;
+    // ---- fused combine ----
+    // The workgroup of the LAST split of this KV head merges the partials of its
+    // query heads, so no second launch is needed. Every split publishes, per query
+    // head, a record {epoch | max} {epoch | sum} after its partial outputs have been
+    // acknowledged; the last split's workgroup waits for all records. Workgroups are
+    // dispatched in index order and the others never wait for anything, so whoever
+    // it waits for is already running or done.
+    // A record carries the epoch of the call that wrote it; anything else (an
+    // uninitialised workspace, an earlier call) reads as "not arrived", so the
+    // workspace needs no clearing. The combiner zeroes the records again so that a
+    // graph replay of this very call (same epoch) starts clean.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
     __syncthreads();
-    // A flag holds the epoch of the call that set it; anything else (an
-    // uninitialised workspace, an earlier call) reads as "not arrived", so the
-    // workspace needs no clearing. The combiner zeroes the flags again so that
-    // a graph replay of this very call (same epoch) starts clean.
-    unsigned long long* flags = a.arrivals + (int64_t)kvh * a.num_splits;
-    if (split != a.num_splits - 1) {
-        if (threadIdx.x == 0) __hip_atomic_store(flags + split, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return;
+    const int S = a.num_splits;
+    const unsigned long long tag = a.epoch & 0xffffffffull;
+    if (threadIdx.x < a.group) {
+        const int h = threadIdx.x;
+        unsigned long long* rec = a.records + ((int64_t)(kvh * a.group + h) * S + split) * 2;
+        const unsigned long long m_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h]);
+        const unsigned long long l_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h + 1]);
+        __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(rec + 1, tag | (l_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __shared__ int s_all_arrived;
-    if (wave == 0) {
+    if (split != S - 1) return;
+
+    __syncthreads();  // s_fin has been read: the merge area may be reused below
+    float* s_w = reinterpret_cast<float*>(smem);                                     // [G][kMaxSplits] weights
+    float* s_den = reinterpret_cast<float*>(smem + G * kMaxSplits * sizeof(float));  // [G] denominators
+    int* s_ok = reinterpret_cast<int*>(s_den + G);                                   // [NW] every record seen
+    bool wave_ok = true;
+    // One wave per head: wait for the head's records, then M = max m_s, weights
+    // e^(m_s - M), denominator sum l_s * weight -- all from the polled registers.
+    for (int h = wave; h < a.group; h += NW) {
+        unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
+        constexpr int kSlots = kMaxSplits / 64;
+        float m_reg[kSlots], l_reg[kSlots];
         bool ok = false;
-        // Bounded wait: every wave leaves this loop even if a flag never shows up
-        // (the result is then marked invalid below instead of hanging the GPU).
+        // Bounded wait: every wave leaves this loop even if a record never shows up
+        // (the result is then poisoned below instead of hanging the GPU).
         for (int spin = 0; spin < kMaxSpins; ++spin) {
             ok = true;
-            for (int sp = lane; sp < a.num_splits - 1; sp += 64)
-                ok = ok && (__hip_atomic_load(flags + sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch);
+#pragma unroll
+            for (int j = 0; j < kSlots; ++j) {
+                const int sp = lane + 64 * j;
+                m_reg[j] = -INFINITY;
+                l_reg[j] = 0.0f;
+                if (sp < S) {
+                    const unsigned long long r0 = __hip_atomic_load(rec + 2 * sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const unsigned long long r1 = __hip_atomic_load(rec + 2 * sp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ok = ok && (r0 & 0xffffffffull) == tag && (r1 & 0xffffffffull) == tag;
+                    m_reg[j] = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
+                    l_reg[j] = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
+                }
+            }
             if (__all(ok)) break;
-            __builtin_amdgcn_s_sleep(8);
+            __builtin_amdgcn_s_sleep(4);
         }
-        for (int sp = lane; sp < a.num_splits - 1; sp += 64)
-            __hip_atomic_store(flags + sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (lane == 0) s_all_arrived = __all(ok) ? 1 : 0;
-    }
-    __syncthreads();
-    const bool all_arrived = s_all_arrived != 0;
-    // Every other workgroup's partials were acknowledged before its flag was
-    // set; read them with device-coherent loads.
-    auto coherent = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-
-    float* s_w = reinterpret_cast<float*>(smem);                                   // [G][kMaxSplits] weights
-    float* s_den = reinterpret_cast<float*>(smem + G * kMaxSplits * sizeof(float));  // [G] denominators
-    const int S = a.num_splits;
-    const float* ws_m = a.ws + (int64_t)a.n_q * S * kHeadDim;
-    const float* ws_l = a.ws + (int64_t)a.n_q * S * (kHeadDim + 1);
-    // One wave per head: M = max m_s, weights e^(m_s - M), denominator sum l_s * weight.
-    for (int h = wave; h < a.group; h += NW) {
-        const int64_t row = (int64_t)(kvh * a.group + h) * S;
+        wave_ok = wave_ok && __all(ok);
         float mx = -INFINITY;
-        for (int sp = lane; sp < S; sp += 64) mx = fmaxf(mx, coherent(ws_m + row + sp));
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) mx = fmaxf(mx, m_reg[j]);
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
         float den = 0.0f;
-        for (int sp = lane; sp < S; sp += 64) {
-            const float m = coherent(ws_m + row + sp);
-            const float f = (m == -INFINITY) ? 0.0f : fast_exp2(m - mx);
-            s_w[h * kMaxSplits + sp] = f;
-            den += coherent(ws_l + row + sp) * f;
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            const int sp = lane + 64 * j;
+            if (sp < S) {
+                const float f = (m_reg[j] == -INFINITY) ? 0.0f : fast_exp2(m_reg[j] - mx);
+                s_w[h * kMaxSplits + sp] = f;
+                den += l_reg[j] * f;
+                __hip_atomic_store(rec + 2 * sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(rec + 2 * sp + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) den += __shfl_xor(den, d);
         if (lane == 0) s_den[h] = den;
     }
+    if (lane == 0) s_ok[wave] = wave_ok ? 1 : 0;
     __syncthreads();
+    bool all_arrived = true;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) all_arrived = all_arrived && s_ok[w] != 0;
+    // Every other workgroup's partials were acknowledged before its records were
+    // written; read them with device-coherent loads.
+    auto coherent = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
         const int h = idx >> 7;
         const int d = idx & (kHeadDim - 1);
@@ -533,13 +580,13 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
     ka.ws = static_cast<float*>(args.workspace);
     ka.out = static_cast<uint16_t*>(args.output);
     ka.out_f32 = args.output_f32;
-    ka.arrivals = nullptr;
+    ka.records = nullptr;
     ka.epoch = 0;
     if (plan.path == LLMI_PATH_SPLIT_FUSED) {
-        // Arrival flags sit behind the partials in the workspace.
-        const size_t partial_bytes = (size_t)args.head_num * plan.num_splits * (args.head_dim + 2) * sizeof(float);
-        ka.arrivals = reinterpret_cast<unsigned long long*>(static_cast<char*>(args.workspace) +
-                                                            ((partial_bytes + 15) & ~(size_t)15));
+        // Arrival records sit behind the partial outputs in the workspace.
+        const size_t partial_bytes = (size_t)args.head_num * plan.num_splits * args.head_dim * sizeof(float);
+        ka.records = reinterpret_cast<unsigned long long*>(static_cast<char*>(args.workspace) +
+                                                           ((partial_bytes + 15) & ~(size_t)15));
         ka.epoch = next_epoch();
     }
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
