@@ -63,6 +63,23 @@ def make_arena(torch, dev, ctx_list):
     return k, v, q, regions
 
 
+def measured_traffic(ctx_list):
+    """HBM bytes per launch of the decode kernel over the default sweep, as counted by rocprofv3
+    (FETCH_SIZE + WRITE_SIZE, each scaled by a calibration copy): bench.py cannot run the profiler on
+    itself, so it reports the figure of the committed counter summary, and only for the workload that
+    summary was taken on."""
+    if ctx_list != DEFAULT_CTX:
+        return None
+    path = os.path.join(ROOT, "profiles", "mha_decode_kernel_qwen3-4b_ctx1k-32k_hbm_counters.md")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(ctx_list, budget_s=12.0):
     """The CPU oracle (a port of the reference's single-threaded CPU attention path) timed on this
     host on the same shapes: whole sweeps until about `budget_s` seconds have been spent."""
@@ -204,7 +221,7 @@ def main():
         "us_per_layer_mean": round(avg_launch_us, 3),
         "per_ctx": per_ctx,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(ctx_list),
                      "kernel": "mha_decode_kernel", "launches": steps * launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3), "avg_launch_bytes": int(avg_launch_bytes)},
     }
