@@ -118,8 +118,8 @@ def main():
     ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (--gpus %d refused): the path has no multi-GPU "
-              "part; see DESIGN.md for how it would shard." % args.gpus, file=sys.stderr)
+        print("bench.py: this build measures one GPU only (--gpus %d refused): decode attention at batch 1 "
+              "has no multi-GPU part here." % args.gpus, file=sys.stderr)
         return 2
     ctx_list = [int(c) for c in args.ctx.split(",")]
 
