@@ -21,13 +21,16 @@ thread_local std::string g_last_error;
 
 // Context lengths up to this run as one workgroup per KV head; longer ones are
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
-// splits, mha_kernel.cu:507-517; here a split costs a second launch and a
-// workspace round trip, and one workgroup already streams a whole KV head.)
-constexpr int kSinglePassMaxLen = 256;
+// splits, mha_kernel.cu:507-517. Here the split path pays three dependent
+// memory round trips for its combine, about 3 us, while one workgroup streams a
+// whole KV head at 16 tiles in about 7 us: measured crossover between 192 and
+// 256 positions at 32 query / 8 KV heads.)
+constexpr int kSinglePassMaxLen = 240;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).
 constexpr int kTargetGroups = 256;
+constexpr int kMinGroups = 128;
 constexpr int kTile = 16;
 
 inline int pow2_ceil(int x) {
@@ -115,15 +118,23 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p) {
         if (want == 0) {
             // Auto: a few workgroups per CU, at least one tile per wave, and
             // no more splits than the caller's workspace can hold.
-            want = kTargetGroups / n_kv;
-            if (want < 2) want = 2;
-            if (want > kMaxSplits) want = kMaxSplits;
+            // One workgroup per CU for long contexts; for short ones one tile per
+            // wave, but never fewer than kMinGroups workgroups (idle waves cost less
+            // than idle CUs: measured at ctx 256..2048).
+            int target = kTargetGroups / n_kv;
+            if (target < 2) target = 2;
+            if (target > kMaxSplits) target = kMaxSplits;
+            int floor_splits = kMinGroups / n_kv;
+            if (floor_splits < 2) floor_splits = 2;
+            want = ceil_div(tiles, waves);
+            if (want < floor_splits) want = floor_splits;
+            if (want > target) want = target;
+            if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;
             const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
             if (cap < 2) return LLMI_ERR_WORKSPACE;
             if ((size_t)want > cap) want = (int)cap;
             tiles_per_split = ceil_div(tiles, want);
-            if (tiles_per_split < waves) tiles_per_split = waves;
         } else {
             tiles_per_split = ceil_div(tiles, want);
         }

@@ -107,7 +107,7 @@ def test_null_arguments():
 
 
 def test_plan_short_context_is_single_pass():
-    for pos in (0, 15, 16, 127, 255):
+    for pos in (0, 15, 16, 127, 239):
         rc, p = plan(good_args(pos=pos, workspace=0, workspace_bytes=0))  # no workspace needed
         assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1 and p.workspace_needed == 0
         assert p.rows_per_split >= pos + 1 and p.rows_per_split % 16 == 0
