@@ -35,7 +35,7 @@ def algorithmic_bytes(ctx, n_q=N_Q, n_kv=N_KV):
     return 2 * ctx * n_kv * HEAD_DIM * 2 + 2 * n_q * HEAD_DIM * 2
 
 
-def make_arena(torch, dev, ctx_list):
+def make_arena(torch, dev, ctx_list, n_q=N_Q):
     """One K and one V slab; each (ctx, slice) pair owns a distinct region. Values: N(0,1),
     RMS-normalised per 128-wide head vector, rounded to bf16."""
     total_rows = sum(ctx_list) * SLICES
@@ -58,7 +58,7 @@ def make_arena(torch, dev, ctx_list):
         for s in range(SLICES):
             regions[(ctx, s)] = row * KV_DIM  # element offset of a [N_KV][ctx][128] cache
             row += ctx
-    q = torch.randn((N_Q, HEAD_DIM), generator=gen, device=dev)
+    q = torch.randn((n_q, HEAD_DIM), generator=gen, device=dev)
     q = (q * torch.rsqrt((q * q).mean(dim=1, keepdim=True))).to(torch.bfloat16).reshape(-1)
     return k, v, q, regions
 
@@ -80,7 +80,7 @@ def measured_traffic(ctx_list):
     return None
 
 
-def cpu_baseline(ctx_list, budget_s=12.0):
+def cpu_baseline(ctx_list, budget_s=12.0, n_q=N_Q):
     """The CPU oracle (a port of the reference's single-threaded CPU attention path) timed on this
     host on the same shapes: whole sweeps until about `budget_s` seconds have been spent."""
     import numpy as np
@@ -88,7 +88,7 @@ def cpu_baseline(ctx_list, budget_s=12.0):
     from llminfer_amd import synth
     cases = []
     for ctx in ctx_list:
-        c = synth.make_case(1000 + ctx, n_q=N_Q, n_kv=N_KV, ctx=ctx)
+        c = synth.make_case(1000 + ctx, n_q=n_q, n_kv=N_KV, ctx=ctx)
         cases.append(c)
     oracle.lib()
     passes, t_total = 0, 0.0
@@ -99,13 +99,81 @@ def cpu_baseline(ctx_list, budget_s=12.0):
                            c["head_num"], c["head_dim"], c["max_seq_len"])
         t_total += time.perf_counter() - t0
         passes += 1
-    nbytes = sum(algorithmic_bytes(c) for c in ctx_list) * passes
+    nbytes = sum(algorithmic_bytes(c, n_q) for c in ctx_list) * passes
     return {
         "value": round(nbytes / t_total / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": "%d passes of the same ctx sweep %s through the CPU oracle (bf16 inputs widened to fp32), "
                   "%.1f s, %.0f us per layer call on average"
                   % (passes, ctx_list, t_total, t_total / (passes * len(ctx_list)) * 1e6),
     }
+
+
+def run_stack(args, ctx):
+    """BASELINE config 4: the attention part of a 36-layer decode step at a fixed position, as one HIP graph."""
+    import numpy as np
+    from llminfer_amd import _binding as B
+    from llminfer_amd import synth
+    host = ctypes.CDLL(os.path.join(ROOT, "llminfer_amd", "libllmi_host.so"))
+    host.llmi_host_stack_create.restype = ctypes.c_void_p
+    host.llmi_host_stack_create.argtypes = [ctypes.c_int32] * 5
+    host.llmi_host_stack_ptr.restype = ctypes.c_void_p
+    host.llmi_host_stack_ptr.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+    host.llmi_host_stack_build_sincos.argtypes = [ctypes.c_void_p]
+    host.llmi_host_stack_run.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+    host.llmi_host_stack_capture.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+    host.llmi_host_stack_replay.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_float)]
+    host.llmi_host_stack_destroy.argtypes = [ctypes.c_void_p]
+    host.llmi_host_last_error.restype = ctypes.c_char_p
+    layers, n_q, msl, pos = args.stack, args.heads, ctx + 8, ctx
+    st = host.llmi_host_stack_create(layers, msl, n_q, N_KV, args.layout)
+    if not st:
+        print("bench.py: " + host.llmi_host_last_error().decode(), file=sys.stderr)
+        return 1
+
+    def up(ptr, arr):
+        arr = np.ascontiguousarray(arr)
+        B.check(B.lib().llmi_hip_memcpy(ptr, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes, 1, None, 1), "upload")
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(host.llmi_host_last_error().decode())
+
+    ok(host.llmi_host_stack_build_sincos(st))
+    rng = np.random.RandomState(4)
+    rows = rng.standard_normal((msl * N_KV, HEAD_DIM)).astype(np.float32)
+    rows /= np.sqrt((rows * rows).mean(axis=1, keepdims=True))
+    layer_bits = synth.f32_to_bf16_bits(rows).reshape(-1)  # one layer's worth, reused (rolled) for every layer
+    for which in (0, 1):
+        base = host.llmi_host_stack_ptr(st, which, 0)
+        for l in range(layers):
+            up(base + l * layer_bits.nbytes, np.roll(layer_bits, 128 * (l + 17 * which)))
+    for l in range(layers):
+        up(host.llmi_host_stack_ptr(st, 2, l), synth.f32_to_bf16_bits(rng.standard_normal(n_q * HEAD_DIM).astype(np.float32)))
+        up(host.llmi_host_stack_ptr(st, 3, l), synth.f32_to_bf16_bits(rng.standard_normal(KV_DIM).astype(np.float32)))
+        up(host.llmi_host_stack_ptr(st, 4, l), synth.f32_to_bf16_bits(rng.standard_normal(KV_DIM).astype(np.float32)))
+        up(host.llmi_host_stack_ptr(st, 5, l),
+           synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * HEAD_DIM)).astype(np.float32)))
+    ok(host.llmi_host_stack_run(st, pos, 1))
+    ok(host.llmi_host_stack_capture(st, pos, 1))
+    ms = ctypes.c_float()
+    ok(host.llmi_host_stack_replay(st, max(1, args.warmup), ctypes.byref(ms)))
+    ok(host.llmi_host_stack_replay(st, args.steps, ctypes.byref(ms)))
+    us_token = ms.value * 1e3 / args.steps
+    per_layer = algorithmic_bytes(pos + 1, n_q) + 23552  # + QK-Norm/RoPE/append traffic per layer
+    gbs = layers * per_layer / (us_token * 1e-6) / 1e9
+    host.llmi_host_stack_destroy(st)
+    print(json.dumps({
+        "metric": "attention stack of one decode step, us per token", "value": round(us_token, 2), "unit": "us/token",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us_token / 1e3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%d layers x (fused QK-Norm + RoPE + K/V append, GQA decode attention), %d Q / 8 KV "
+                               "heads, ctx %d + 1 new token, one HIP graph per token, %s layout"
+                               % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major")},
+        "us_per_layer": round(us_token / layers, 3),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+    }))
+    return 0
 
 
 def main():
@@ -116,12 +184,19 @@ def main():
     ap.add_argument("--ctx", type=str, default=",".join(map(str, DEFAULT_CTX)))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
+    ap.add_argument("--heads", type=int, default=N_Q, help="query heads (32 = Qwen3-4B, 64 = Qwen3-32B head layout)")
+    ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
+                    help="instead of the sweep: LAYERS layers of (QK-Norm + RoPE + append, attention) at --ctx (one "
+                         "value) + 1 new token, captured into one HIP graph; reports us per token")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus %d refused): decode attention at batch 1 "
               "has no multi-GPU part here." % args.gpus, file=sys.stderr)
         return 2
     ctx_list = [int(c) for c in args.ctx.split(",")]
+    n_q = args.heads
+    if args.stack:
+        return run_stack(args, ctx_list[0])
 
     import torch
     from llminfer_amd import _binding as B
@@ -134,15 +209,15 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    k, v, q, regions = make_arena(torch, dev, ctx_list)
-    out = torch.empty(N_Q * HEAD_DIM, dtype=torch.bfloat16, device=dev)
-    ws = torch.empty(ops.workspace_bytes(N_Q, HEAD_DIM, max(ctx_list)) // 4, dtype=torch.float32, device=dev)
+    k, v, q, regions = make_arena(torch, dev, ctx_list, n_q)
+    out = torch.empty(n_q * HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(ops.workspace_bytes(n_q, HEAD_DIM, max(ctx_list)) // 4, dtype=torch.float32, device=dev)
     esz = 2
 
     def call_args(ctx, s):
         off = regions[(ctx, s)] * esz
         return ops.make_mha_args(q, k.data_ptr() + off, v.data_ptr() + off, out, ws, layer_id=0, pos=ctx - 1,
-                                 kv_dim=KV_DIM, kv_mul=N_Q // N_KV, head_num=N_Q, head_dim=HEAD_DIM,
+                                 kv_dim=KV_DIM, kv_mul=n_q // N_KV, head_num=n_q, head_dim=HEAD_DIM,
                                  max_seq_len=ctx, kv_layout=args.layout)
 
     plans = {ctx: ops.mha_plan(call_args(ctx, 0)) for ctx in ctx_list}
@@ -185,7 +260,7 @@ def main():
     ms = time_graph(g_all, steps // SLICES)
     torch.cuda.synchronize()
     ms_per_step = ms / steps
-    step_bytes = sum(algorithmic_bytes(c) for c in ctx_list)
+    step_bytes = sum(algorithmic_bytes(c, n_q) for c in ctx_list)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     launches_per_step = len(ctx_list)  # every call of the sweep is one launch of the decode kernel
 
@@ -199,7 +274,7 @@ def main():
         t = time_graph(g, n // SLICES)
         torch.cuda.synchronize()
         us = t * 1e3 / n
-        gbs = algorithmic_bytes(ctx) / (us * 1e-6) / 1e9
+        gbs = algorithmic_bytes(ctx, n_q) / (us * 1e-6) / 1e9
         p = plans[ctx]
         per_ctx.append({"ctx": ctx, "us_per_layer": round(us, 3), "GBps": round(gbs, 1),
                         "frac_peak": round(gbs / HBM_PEAK_GBS, 4), "path": p.path, "splits": p.num_splits,
@@ -213,20 +288,22 @@ def main():
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "Qwen3-4B layer shape (32 Q / 8 KV heads, head_dim 128), batch 1, one decode-"
+        "config": {"workload": "%s layer shape (%d Q / 8 KV heads, head_dim 128), batch 1, one decode-"
                                "attention layer call per context in %s per step, bf16 KV cache, %s layout, "
                                "HIP-graph replays over %d rotating KV slices per context"
-                               % (ctx_list, "head-major" if args.layout == 1 else "position-major", SLICES),
+                               % ("Qwen3-4B" if n_q == 32 else "Qwen3-32B-heads" if n_q == 64 else "custom", n_q,
+                                  ctx_list, "head-major" if args.layout == 1 else "position-major", SLICES),
                    "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout},
         "us_per_layer_mean": round(avg_launch_us, 3),
         "per_ctx": per_ctx,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(ctx_list),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(ctx_list) if n_q == N_Q else None,
                      "kernel": "mha_decode_kernel", "launches": steps * launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3), "avg_launch_bytes": int(avg_launch_bytes)},
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(ctx_list)
+        result["cpu_baseline"] = cpu_baseline(ctx_list, n_q=n_q)
     print(json.dumps(result))
     return 0
 
