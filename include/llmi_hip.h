@@ -13,6 +13,8 @@
  *                                 (registry slot kernel_interface.h:168-183,
  *                                 kernel_interface.cpp:181-190; caller
  *                                 code/source/op/mha.cpp:54-56)
+ *   llmi_hip_mha_decode_append    the pair fused_qk_norm_rope_kernel_cu + mha_kernel_cu as
+ *                                 the layer loop issues it, code/source/model/qwen3_fused.cpp:524-548
  *   llmi_hip_mha_workspace_bytes  the KVSplitOutput buffer sizing
  *                                 code/source/model/qwen3_fused.cpp:502-503
  *   llmi_hip_mha_plan             the dispatch arithmetic inside mha_kernel_cu
@@ -113,6 +115,25 @@ int llmi_hip_mha_plan(const llmi_mha_args* args, llmi_mha_plan* plan);
  * under stream capture. The workspace needs no initialisation. Two calls that
  * share a workspace must not overlap in time. */
 int llmi_hip_mha_decode(const llmi_mha_args* args);
+
+typedef struct llmi_mha_append_args {
+    llmi_mha_args mha;        /* as for llmi_hip_mha_decode, except: mha.query is the RAW query of the new
+                                 token (before QK-Norm), and the caches are written at (layer_id, pos)  */
+    const void* key_new;      /* device bf16 [kv_dim]: the new token's raw K row                        */
+    const void* value_new;    /* device bf16 [kv_dim]: the new token's V row                            */
+    const void* norm_weight;  /* device bf16 [2*128]: q_norm then k_norm                                */
+    const float* sin_cache;   /* device fp32 [max_seq_len][64]                                          */
+    const float* cos_cache;   /* device fp32 [max_seq_len][64]                                          */
+    float eps;                /* 1e-6 in the reference                                                  */
+} llmi_mha_append_args;
+
+/* llmi_hip_qk_norm_rope_append followed by llmi_hip_mha_decode, as ONE kernel launch: the query group and
+ * the new K row are normalised + rotated inside the attention kernel, the K and V rows of position `pos`
+ * are stored to the cache (either layout) and used from registers. The normalised query is not written
+ * back. Replaces the back-to-back pair fused_qk_norm_rope + mha of the reference's layer loop
+ * (code/source/model/qwen3_fused.cpp:524-548; kernels rmsnorm_kernel.cu:248-290, mha_kernel.cu:440-529).
+ * The separate-combine path (LLMI_PATH_SPLIT) and 8 waves per workgroup are not available here. */
+int llmi_hip_mha_decode_append(const llmi_mha_append_args* args);
 
 /* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len);

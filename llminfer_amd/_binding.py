@@ -34,6 +34,13 @@ class MhaArgs(ctypes.Structure):
     ]
 
 
+class MhaAppendArgs(ctypes.Structure):
+    _fields_ = [
+        ("mha", MhaArgs), ("key_new", c_void_p), ("value_new", c_void_p), ("norm_weight", c_void_p),
+        ("sin_cache", c_void_p), ("cos_cache", c_void_p), ("eps", ctypes.c_float),
+    ]
+
+
 class MhaPlan(ctypes.Structure):
     _fields_ = [
         ("path", c_i32), ("num_splits", c_i32), ("rows_per_split", c_i32),
@@ -66,6 +73,7 @@ BACKING_FREE_FN = ctypes.CFUNCTYPE(ctypes.c_int, c_void_p, c_void_p)
 SYMBOLS = {
     "llmi_hip_mha_plan": (ctypes.c_int, [ctypes.POINTER(MhaArgs), ctypes.POINTER(MhaPlan)]),
     "llmi_hip_mha_decode": (ctypes.c_int, [ctypes.POINTER(MhaArgs)]),
+    "llmi_hip_mha_decode_append": (ctypes.c_int, [ctypes.POINTER(MhaAppendArgs)]),
     "llmi_hip_mha_workspace_bytes": (c_size_t, [c_i32, c_i32, c_i32]),
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),
     "llmi_hip_sincos_table": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_void_p]),

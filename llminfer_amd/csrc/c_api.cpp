@@ -184,6 +184,21 @@ int llmi_hip_mha_decode(const llmi_mha_args* args) {
     return launch_mha_decode(*args, plan);
 }
 
+int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
+    if (!args) return LLMI_ERR_NULL_POINTER;
+    if (!args->key_new || !args->value_new || !args->norm_weight || !args->sin_cache || !args->cos_cache)
+        return LLMI_ERR_NULL_POINTER;
+    const void* ptrs[] = {args->key_new, args->value_new, args->norm_weight, args->sin_cache, args->cos_cache};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
+    if (!(args->eps >= 0.0f)) return LLMI_ERR_INVALID_ARG;
+    if (args->mha.force_path == LLMI_PATH_SPLIT || args->mha.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
+    llmi_mha_plan plan;
+    if (int rc = make_plan(&args->mha, &plan)) return rc;
+    if (plan.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
+    return launch_mha_decode(args->mha, plan, args);
+}
+
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len) {
     if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     int splits = (max_seq_len + kTile - 1) / kTile;

@@ -39,7 +39,8 @@ void DecodeStack::build_sincos() {
     synchronize();
 }
 
-void DecodeStack::enqueue(int32_t pos, bool with_qk_norm_rope) {
+void DecodeStack::enqueue(int32_t pos, int32_t mode) {
+    const bool with_qk_norm_rope = mode == kSeparateQkNormRope;
     const AttentionConfig& c = config_;
     tensor::Tensor& kc = buffers_->get_buffer(ModelBufferType::KeyCache);
     tensor::Tensor& vc = buffers_->get_buffer(ModelBufferType::ValueCache);
@@ -91,12 +92,26 @@ void DecodeStack::enqueue(int32_t pos, bool with_qk_norm_rope) {
         m.num_splits = o.num_splits;
         m.waves_per_group = o.waves_per_group;
         m.stream = stream();
-        const int rc = llmi_hip_mha_decode(&m);
-        if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_mha_decode: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
+        int rc;
+        if (mode == kFusedAppend) {
+            llmi_mha_append_args f{};
+            f.mha = m;
+            f.mha.query = query_raw(layer);
+            f.key_new = key_raw(layer);
+            f.value_new = value_raw(layer);
+            f.norm_weight = norm_weight(layer);
+            f.sin_cache = buffers_->get_buffer(ModelBufferType::SinCache).ptr<float>();
+            f.cos_cache = buffers_->get_buffer(ModelBufferType::CosCache).ptr<float>();
+            f.eps = 1e-6f;
+            rc = llmi_hip_mha_decode_append(&f);
+        } else {
+            rc = llmi_hip_mha_decode(&m);
+        }
+        if (rc != LLMI_OK) LLMI_FATAL("decode attention: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
     }
 }
 
-void DecodeStack::capture(int32_t pos, bool with_qk_norm_rope) {
+void DecodeStack::capture(int32_t pos, int32_t mode) {
     if (graph_exec_) {
         HIP_OK(hipGraphExecDestroy(graph_exec_));
         graph_exec_ = nullptr;
@@ -107,7 +122,7 @@ void DecodeStack::capture(int32_t pos, bool with_qk_norm_rope) {
     }
     HIP_OK(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
     try {
-        enqueue(pos, with_qk_norm_rope);
+        enqueue(pos, mode);
     } catch (...) {
         hipGraph_t dead = nullptr;
         (void)hipStreamEndCapture(stream(), &dead);

@@ -33,10 +33,13 @@ public:
     uint16_t* output(int32_t layer) { return outputs_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.dim()); }
 
     void build_sincos();
+    // What one layer issues: attention alone on the raw query (0), the QK-Norm + RoPE + append kernel
+    // followed by attention (1, the reference's sequence), or both fused into one launch (2).
+    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2 };
     // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
-    void enqueue(int32_t pos, bool with_qk_norm_rope);
-    // Captures enqueue(pos) into a graph (replacing an earlier one).
-    void capture(int32_t pos, bool with_qk_norm_rope);
+    void enqueue(int32_t pos, int32_t mode);
+    // Captures enqueue(pos, mode) into a graph (replacing an earlier one).
+    void capture(int32_t pos, int32_t mode);
     // Replays the captured graph `times` times; returns the elapsed milliseconds (HIP events on the stream).
     float replay(int32_t times);
     void synchronize();

@@ -74,13 +74,13 @@ int llmi_host_stack_build_sincos(llmi_host_stack* s) { return guarded([&] { s->i
 
 int llmi_host_stack_run(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope) {
     return guarded([&] {
-        s->impl->enqueue(pos, with_qk_norm_rope != 0);
+        s->impl->enqueue(pos, with_qk_norm_rope);
         s->impl->synchronize();
     });
 }
 
 int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope) {
-    return guarded([&] { s->impl->capture(pos, with_qk_norm_rope != 0); });
+    return guarded([&] { s->impl->capture(pos, with_qk_norm_rope); });
 }
 
 int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms) {

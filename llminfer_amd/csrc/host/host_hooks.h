@@ -22,6 +22,7 @@ void llmi_host_stack_destroy(llmi_host_stack* s);
  * 5 norm weight, 6 output of `layer`, 7 sin table, 8 cos table, 9 normalised query buffer. Device pointers. */
 void* llmi_host_stack_ptr(llmi_host_stack* s, int32_t which, int32_t layer);
 int llmi_host_stack_build_sincos(llmi_host_stack* s);
+/* with_qk_norm_rope: 0 attention only, 1 separate QK-Norm/RoPE/append kernel + attention, 2 both fused */
 int llmi_host_stack_run(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);      /* eager + synchronise */
 int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);
 int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms);

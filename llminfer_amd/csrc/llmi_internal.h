@@ -22,7 +22,8 @@ int check_launch();
 // A fresh 48-bit tag per decode call (never 0), for the arrival cells of the fused combine.
 unsigned long long next_epoch();
 
-int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan);
+// `append` non-null: the fused QK-Norm + RoPE + K/V append variant.
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append = nullptr);
 int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);
 int launch_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,
                         hipStream_t stream);

@@ -141,9 +141,80 @@ struct KernelArgs {
     int32_t num_splits;
     int32_t rows_per_split;  // multiple of kTile
     float scale_log2e;       // log2(e) / sqrt(head_dim)
+    // Fused append (APPEND kernels only): q is the raw query; the new token's K
+    // row is normalised + rotated, its V row copied, both stored at position
+    // seq_len-1 of the cache and used from registers.
+    const uint16_t* k_new;   // [n_kv][128] raw
+    const uint16_t* v_new;   // [n_kv][128]
+    const uint16_t* norm_w;  // [2][128]: q_norm, k_norm
+    const float* sin_row;    // [64] of this position
+    const float* cos_row;
+    uint16_t* k_slot;        // cache address of (layer, seq_len-1, kv_head 0)
+    uint16_t* v_slot;
+    int64_t slot_head_stride;
+    float eps;
 };
 
-template <int G, int NW, int NSTAGE>
+// RMSNorm * weight + half-rotation RoPE of one 128-wide row, for the lane's 32
+// elements in the MFMA operand layout (dims (j*4+kg)*8 .. +8, j = 0..3), rounded
+// to bf16. The four lanes that share a row (kg = 0..3 of one DPP column) add up
+// the sum of squares with two xor shuffles. Same chain as the stand-alone kernel
+// (x*w*r, then a*cos - b*sin / a*sin + b*cos on the pairs (i, i+64)).
+__device__ __forceinline__ void norm_rope_row(const uint16_t* row, const uint16_t* w, const float* sin_row,
+                                              const float* cos_row, float eps, int kg, u32x4 (&out)[4]) {
+    float x[4][8], wt[4][8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32x4 xr = *reinterpret_cast<const u32x4*>(row + (j * 4 + kg) * 8);
+        const u32x4 wr = *reinterpret_cast<const u32x4*>(w + (j * 4 + kg) * 8);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            x[j][2 * c] = bf16_lo(xr[c]);
+            x[j][2 * c + 1] = bf16_hi(xr[c]);
+            wt[j][2 * c] = bf16_lo(wr[c]);
+            wt[j][2 * c + 1] = bf16_hi(wr[c]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
+    }
+    ss += __shfl_xor(ss, 16);
+    ss += __shfl_xor(ss, 32);
+    const float r = 1.0f / sqrtf(ss / (float)kHeadDim + eps);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        float sn[8], cs[8];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const f32x4 s4 = *reinterpret_cast<const f32x4*>(sin_row + (j * 4 + kg) * 8 + 4 * c);
+            const f32x4 c4 = *reinterpret_cast<const f32x4*>(cos_row + (j * 4 + kg) * 8 + 4 * c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                sn[4 * c + e] = s4[e];
+                cs[4 * c + e] = c4[e];
+            }
+        }
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t pl = 0, ph = 0;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int e = 2 * c + half;
+                const float av = x[j][e] * wt[j][e] * r;
+                const float bv = x[j + 2][e] * wt[j + 2][e] * r;
+                pl |= (uint32_t)f32_to_bf16(av * cs[e] - bv * sn[e]) << (16 * half);
+                ph |= (uint32_t)f32_to_bf16(av * sn[e] + bv * cs[e]) << (16 * half);
+            }
+            lo[c] = pl;
+            hi[c] = ph;
+        }
+        out[j] = u32x4{lo[0], lo[1], lo[2], lo[3]};
+        out[j + 2] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    }
+}
+
+template <int G, int NW, int NSTAGE, bool APPEND>
 __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
@@ -162,12 +233,27 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     u32x4 qb[4];
     {
         const int hq = kvh * a.group + min(n16, a.group - 1);
-        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim + kg * 8;
+        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim;
         const bool live = n16 < a.group;
+        if constexpr (APPEND) {
+            norm_rope_row(qp, a.norm_w, a.sin_row, a.cos_row, a.eps, kg, qb);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const u32x4 z = *reinterpret_cast<const u32x4*>(qp + j * 32);
-            qb[j] = live ? z : u32x4{0u, 0u, 0u, 0u};
+            for (int j = 0; j < 4; ++j) qb[j] = *reinterpret_cast<const u32x4*>(qp + kg * 8 + j * 32);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qb[j] = live ? qb[j] : u32x4{0u, 0u, 0u, 0u};
+    }
+    // Fused append: the last tile of the last split holds the new token. Its K row
+    // (normalised + rotated here) and V row are used from registers and stored to
+    // the cache by the wave that owns that tile.
+    u32x4 k_fresh[4] = {};
+    u32x4 v_fresh = {0u, 0u, 0u, 0u};
+    const bool holds_new_row = APPEND && split == a.num_splits - 1;
+    if constexpr (APPEND) {
+        if (holds_new_row) {
+            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_row, a.cos_row, a.eps, kg, k_fresh);
+            v_fresh = *reinterpret_cast<const u32x4*>(a.v_new + kvh * kHeadDim + n16 * 8);
         }
     }
 
@@ -295,6 +381,25 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         TileRegs r;
         wait_tiles_in_flight(min(NSTAGE - 1, n_my - 1 - i));
         read_tile(stage, r);
+        if constexpr (APPEND) {
+            const int t = wave + i * NW;
+            if (holds_new_row && t == ntiles - 1) {
+                // Row `fresh` of this tile is the new token; the rows after it are
+                // clamped re-reads of its (still unwritten) cache slot: give them
+                // all the fresh data, the softmax mask drops the extra ones.
+                const int fresh = (nrows - 1) - t * kTile;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r.k[j] = n16 >= fresh ? k_fresh[j] : r.k[j];
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) r.v[q4] = 4 * kg + q4 >= fresh ? v_fresh : r.v[q4];
+                if (n16 == 0) {
+                    uint16_t* kd = a.k_slot + kvh * a.slot_head_stride;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = k_fresh[j];
+                }
+                if (kg == 0) *reinterpret_cast<u32x4*>(a.v_slot + kvh * a.slot_head_stride + n16 * 8) = v_fresh;
+            }
+        }
         if (i + NSTAGE < n_my) issue_tile(wave + (i + NSTAGE) * NW, stage);
         compute_tile(wave + i * NW, r);
         stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
@@ -547,21 +652,26 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
 #endif
 
 template <int G, int NW>
-void launch_decode(const KernelArgs& ka, int n_kv, hipStream_t stream) {
+void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stream) {
     // The LDS-DMA offset register addresses 64 KiB: NW * NSTAGE * 8 KiB must fit.
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= 65536) ? LLMI_STAGES : 65536 / (NW * 8192);
     dim3 grid(ka.num_splits, n_kv);
-    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages>), grid, dim3(NW * 64), 0, stream, ka);
+    if (append) {
+        if constexpr (NW <= 4) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true>), grid, dim3(NW * 64), 0, stream, ka);
+    } else {
+        hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false>), grid, dim3(NW * 64), 0, stream, ka);
+    }
 }
 
 template <int G>
-bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream) {
+bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream) {
+    if (append && nw > 4) return false;
     switch (nw) {
-        case 1: launch_decode<G, 1>(ka, n_kv, stream); return true;
-        case 2: launch_decode<G, 2>(ka, n_kv, stream); return true;
-        case 4: launch_decode<G, 4>(ka, n_kv, stream); return true;
+        case 1: launch_decode<G, 1>(ka, n_kv, append, stream); return true;
+        case 2: launch_decode<G, 2>(ka, n_kv, append, stream); return true;
+        case 4: launch_decode<G, 4>(ka, n_kv, append, stream); return true;
         case 8:
-            if constexpr (G <= 8) { launch_decode<G, 8>(ka, n_kv, stream); return true; }
+            if constexpr (G <= 8) { launch_decode<G, 8>(ka, n_kv, append, stream); return true; }
             return false;
         default: return false;
     }
@@ -569,11 +679,11 @@ bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream
 
 }  // namespace
 
-int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append) {
     const int n_kv = args.kv_dim / args.head_dim;
     const int64_t layer_off = (int64_t)args.layer_id * args.max_seq_len * args.kv_dim;
 
-    KernelArgs ka;
+    KernelArgs ka{};
     ka.q = static_cast<const uint16_t*>(args.query);
     ka.k = static_cast<const uint16_t*>(args.key_cache) + layer_off;
     ka.v = static_cast<const uint16_t*>(args.value_cache) + layer_off;
@@ -589,12 +699,15 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
                                                            ((partial_bytes + 15) & ~(size_t)15));
         ka.epoch = next_epoch();
     }
+    int64_t slot_off;
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
         ka.row_stride = args.kv_dim;
         ka.head_stride = args.head_dim;
+        slot_off = (int64_t)args.pos * args.kv_dim;
     } else {
         ka.row_stride = args.head_dim;
         ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
+        slot_off = (int64_t)args.pos * args.head_dim;
     }
     ka.seq_len = args.pos + 1;
     ka.group = args.kv_mul;
@@ -602,15 +715,27 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan) {
     ka.num_splits = plan.num_splits;
     ka.rows_per_split = plan.rows_per_split;
     ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
+    if (append) {
+        ka.k_new = static_cast<const uint16_t*>(append->key_new);
+        ka.v_new = static_cast<const uint16_t*>(append->value_new);
+        ka.norm_w = static_cast<const uint16_t*>(append->norm_weight);
+        ka.sin_row = append->sin_cache + (int64_t)args.pos * (args.head_dim / 2);
+        ka.cos_row = append->cos_cache + (int64_t)args.pos * (args.head_dim / 2);
+        ka.k_slot = const_cast<uint16_t*>(ka.k) + slot_off;
+        ka.v_slot = const_cast<uint16_t*>(ka.v) + slot_off;
+        ka.slot_head_stride = ka.head_stride;
+        ka.eps = append->eps;
+    }
 
     hipStream_t stream = static_cast<hipStream_t>(args.stream);
+    const bool ap = append != nullptr;
     bool ok = false;
     switch (plan.group_pad) {
-        case 1: ok = launch_decode_nw<1>(ka, n_kv, plan.waves_per_group, stream); break;
-        case 2: ok = launch_decode_nw<2>(ka, n_kv, plan.waves_per_group, stream); break;
-        case 4: ok = launch_decode_nw<4>(ka, n_kv, plan.waves_per_group, stream); break;
-        case 8: ok = launch_decode_nw<8>(ka, n_kv, plan.waves_per_group, stream); break;
-        case 16: ok = launch_decode_nw<16>(ka, n_kv, plan.waves_per_group, stream); break;
+        case 1: ok = launch_decode_nw<1>(ka, n_kv, plan.waves_per_group, ap, stream); break;
+        case 2: ok = launch_decode_nw<2>(ka, n_kv, plan.waves_per_group, ap, stream); break;
+        case 4: ok = launch_decode_nw<4>(ka, n_kv, plan.waves_per_group, ap, stream); break;
+        case 8: ok = launch_decode_nw<8>(ka, n_kv, plan.waves_per_group, ap, stream); break;
+        case 16: ok = launch_decode_nw<16>(ka, n_kv, plan.waves_per_group, ap, stream); break;
         default: ok = false;
     }
     if (!ok) return LLMI_ERR_INVALID_ARG;

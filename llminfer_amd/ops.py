@@ -104,6 +104,24 @@ def qk_norm_rope_append(query, key_new, value_new, key_cache, value_cache, norm_
     B.check(B.lib().llmi_hip_qk_norm_rope_append(ctypes.byref(a)), "llmi_hip_qk_norm_rope_append")
 
 
+def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos_cache, key_cache, value_cache,
+                      output, workspace, *, eps=1e-6, stream=None, **kw):
+    """QK-Norm + RoPE + K/V append + decode attention as one kernel (llmi_hip_mha_decode_append)."""
+    for name, t in (("query_raw", query_raw), ("key_new", key_new), ("value_new", value_new),
+                    ("norm_weight", norm_weight), ("key_cache", key_cache), ("value_cache", value_cache),
+                    ("output", output)):
+        _check_dev(name, t, _BF16_DTYPES)
+    for name, t in (("sin_cache", sin_cache), ("cos_cache", cos_cache), ("workspace", workspace),
+                    ("output_f32", kw.get("output_f32"))):
+        _check_dev(name, t, (torch.float32,))
+    a = B.MhaAppendArgs()
+    a.mha = make_mha_args(query_raw, key_cache, value_cache, output, workspace, stream=_stream_handle(stream), **kw)
+    a.key_new, a.value_new, a.norm_weight = _ptr(key_new), _ptr(value_new), _ptr(norm_weight)
+    a.sin_cache, a.cos_cache, a.eps = _ptr(sin_cache), _ptr(cos_cache), eps
+    B.check(B.lib().llmi_hip_mha_decode_append(ctypes.byref(a)), "llmi_hip_mha_decode_append")
+    return output
+
+
 def sincos_table(head_dim, max_seq_len, device="cuda", stream=None):
     sin = torch.empty((max_seq_len, head_dim // 2), dtype=torch.float32, device=device)
     cos = torch.empty_like(sin)

@@ -146,6 +146,59 @@ def test_attention_after_append_uses_the_new_row(oracle, dev):
     assert_parity(from_dev_bf16(out), ref, "append + attention")
 
 
+@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
+@pytest.mark.parametrize("n_q,n_kv,ctx,path,splits", [
+    (32, 8, 600, B.PATH_AUTO, 0), (32, 8, 4096, B.PATH_AUTO, 0), (32, 8, 100, B.PATH_AUTO, 0),
+    (32, 8, 0, B.PATH_AUTO, 0), (32, 8, 15, B.PATH_SINGLE_PASS, 0), (32, 8, 16, B.PATH_SINGLE_PASS, 0),
+    (32, 8, 1023, B.PATH_SPLIT_FUSED, 7), (32, 8, 1024, B.PATH_SPLIT_FUSED, 64), (64, 8, 777, B.PATH_AUTO, 0),
+    (16, 8, 300, B.PATH_AUTO, 0), (12, 4, 333, B.PATH_SPLIT_FUSED, 5),
+])
+def test_fused_append_attention(oracle, dev, layout, n_q, n_kv, ctx, path, splits):
+    """llmi_hip_mha_decode_append (norm + rope + append + attention in one launch) against the oracle chain:
+    normalise q and the new K row, put K/V at `pos`, attend over 0..pos; the cache rows it must have written
+    are checked too, and nothing else in the caches may change. ctx = cached positions before the new token."""
+    rng = np.random.RandomState(ctx + n_q)
+    d, msl, pos, kv_dim = 128, ctx + 3, ctx, n_kv * 128
+    case = synth.make_case(500 + ctx, n_q=n_q, n_kv=n_kv, ctx=max(ctx, 1), max_seq_len=msl)
+    k0, v0 = case["k"].copy(), case["v"].copy()
+    k0[0, ctx:] = 0x7FC0  # rows from the new position on are NaN patterns until written
+    v0[0, ctx:] = 0x7FC0
+    q_raw = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+    k_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    v_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+    sin_o, cos_o = oracle.sincos_table(d, msl)
+    q_n = oracle.qk_norm_rope(q_raw, w[:d], sin_o[pos], cos_o[pos])
+    k_n = oracle.qk_norm_rope(k_new, w[d:], sin_o[pos], cos_o[pos])
+    k_ref, v_ref = k0.copy(), v0.copy()
+    k_ref[0, pos] = k_n.reshape(-1)
+    v_ref[0, pos] = v_new.reshape(-1)
+    ref = oracle.mha_cpu(q_n.reshape(-1), k_ref, v_ref, 0, pos, kv_dim, n_q // n_kv, n_q, d, msl)
+
+    hm = layout == B.KV_LAYOUT_HEAD_MAJOR
+    k_d = to_dev(synth.to_head_major(k0, n_kv) if hm else k0, dev)
+    v_d = to_dev(synth.to_head_major(v0, n_kv) if hm else v0, dev)
+    out = torch.zeros(n_q * d, dtype=torch.int16, device=dev)
+    ws = torch.full((ops.workspace_bytes(n_q, d, msl) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    sin_d, cos_d = ops.sincos_table(d, msl, dev)
+    ops.mha_decode_append(to_dev(q_raw.reshape(-1), dev), to_dev(k_new.reshape(-1), dev),
+                          to_dev(v_new.reshape(-1), dev), to_dev(w, dev), sin_d, cos_d, k_d, v_d, out, ws,
+                          layer_id=0, pos=pos, kv_dim=kv_dim, kv_mul=n_q // n_kv, head_num=n_q, head_dim=d,
+                          max_seq_len=msl, kv_layout=layout, force_path=path, num_splits=splits)
+    torch.cuda.synchronize()
+    assert_parity(from_dev_bf16(out), ref, "fused append ctx=%d" % ctx)
+    kc = k_d.cpu().numpy().view(np.uint16)
+    vc = v_d.cpu().numpy().view(np.uint16)
+    if hm:
+        kc = np.ascontiguousarray(kc.transpose(0, 2, 1, 3)).reshape(1, msl, kv_dim)
+        vc = np.ascontiguousarray(vc.transpose(0, 2, 1, 3)).reshape(1, msl, kv_dim)
+    _bf16_close(kc[0, pos].reshape(n_kv, d), k_n, "appended key row")
+    assert np.array_equal(vc[0, pos], v_new.reshape(-1))
+    keep = np.ones(msl, dtype=bool)
+    keep[pos] = False
+    assert np.array_equal(kc[0, keep], k0[0, keep]) and np.array_equal(vc[0, keep], v0[0, keep])
+
+
 def test_default_pool_on_device(dev):
     lib = B.lib()
     a = lib.llmi_hip_pool_alloc(4)
@@ -244,7 +297,16 @@ def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout):
 
         H.ok(H.L.llmi_host_stack_run(stack, pos, 1))
         check("eager")
-        H.ok(H.L.llmi_host_stack_capture(stack, pos, 1))
+        k_after = _download(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up.shape, np.uint16)
+        _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up)  # forget the appended rows
+        _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), v_up)
+        for l in range(layers):
+            _upload(H.L.llmi_host_stack_ptr(stack, 6, l), np.zeros(n_q * d, dtype=np.uint16))
+        H.ok(H.L.llmi_host_stack_run(stack, pos, 2))  # the same step with norm/rope/append fused into attention
+        check("eager fused append")
+        k_fused = _download(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up.shape, np.uint16)
+        assert (k_fused == k_after).mean() > 0.9999  # the appended K rows agree up to rare bf16 rounding flips
+        H.ok(H.L.llmi_host_stack_capture(stack, pos, 2))
         ms = ctypes.c_float()
         for rep in range(3):
             for l in range(layers):  # wipe the outputs between replays
