@@ -153,8 +153,8 @@ def run_stack(args, ctx):
         up(host.llmi_host_stack_ptr(st, 4, l), synth.f32_to_bf16_bits(rng.standard_normal(KV_DIM).astype(np.float32)))
         up(host.llmi_host_stack_ptr(st, 5, l),
            synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * HEAD_DIM)).astype(np.float32)))
-    ok(host.llmi_host_stack_run(st, pos, 1))
-    ok(host.llmi_host_stack_capture(st, pos, 1))
+    ok(host.llmi_host_stack_run(st, pos, args.stack_mode))
+    ok(host.llmi_host_stack_capture(st, pos, args.stack_mode))
     ms = ctypes.c_float()
     ok(host.llmi_host_stack_replay(st, max(1, args.warmup), ctypes.byref(ms)))
     ok(host.llmi_host_stack_replay(st, args.steps, ctypes.byref(ms)))
@@ -167,8 +167,9 @@ def run_stack(args, ctx):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us_token / 1e3, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%d layers x (fused QK-Norm + RoPE + K/V append, GQA decode attention), %d Q / 8 KV "
-                               "heads, ctx %d + 1 new token, one HIP graph per token, %s layout"
-                               % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major")},
+                               "heads, ctx %d + 1 new token, one HIP graph per token, %s layout, %s"
+                               % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major",
+                                  "one launch per layer" if args.stack_mode == 2 else "two launches per layer")},
         "us_per_layer": round(us_token / layers, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
@@ -188,6 +189,9 @@ def main():
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
                     help="instead of the sweep: LAYERS layers of (QK-Norm + RoPE + append, attention) at --ctx (one "
                          "value) + 1 new token, captured into one HIP graph; reports us per token")
+    ap.add_argument("--stack-mode", type=int, default=2,
+                    help="with --stack: 2 = norm/rope/append fused into the attention launch (default), "
+                         "1 = separate kernel before attention (the reference's sequence)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus %d refused): decode attention at batch 1 "

@@ -227,35 +227,11 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     const int nrows = min(a.rows_per_split, a.seq_len - begin);  // > 0: the host never makes empty splits
     const int ntiles = (nrows + kTile - 1) / kTile;
 
-    // Query group as the MFMA B operand (zero columns beyond the group). The
-    // load itself is unpredicated (padding lanes re-read the last head) so
-    // that it does not force a full wait on the first K/V tile.
-    u32x4 qb[4];
-    {
-        const int hq = kvh * a.group + min(n16, a.group - 1);
-        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim;
-        const bool live = n16 < a.group;
-        if constexpr (APPEND) {
-            norm_rope_row(qp, a.norm_w, a.sin_row, a.cos_row, a.eps, kg, qb);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) qb[j] = *reinterpret_cast<const u32x4*>(qp + kg * 8 + j * 32);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qb[j] = live ? qb[j] : u32x4{0u, 0u, 0u, 0u};
-    }
-    // Fused append: the last tile of the last split holds the new token. Its K row
-    // (normalised + rotated here) and V row are used from registers and stored to
-    // the cache by the wave that owns that tile.
-    u32x4 k_fresh[4] = {};
-    u32x4 v_fresh = {0u, 0u, 0u, 0u};
+    // Filled in below, once the first tiles are on their way.
+    u32x4 qb[4];                       // query group, MFMA B operand
+    u32x4 k_fresh[4] = {};             // append variant: the new token's K row (operand layout) ...
+    u32x4 v_fresh = {0u, 0u, 0u, 0u};  // ... and V row chunk
     const bool holds_new_row = APPEND && split == a.num_splits - 1;
-    if constexpr (APPEND) {
-        if (holds_new_row) {
-            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_row, a.cos_row, a.eps, kg, k_fresh);
-            v_fresh = *reinterpret_cast<const u32x4*>(a.v_new + kvh * kHeadDim + n16 * 8);
-        }
-    }
 
     // Wave-uniform 64-bit bases of this split; lanes add 32-bit byte offsets
     // (scalar-base + vector-offset addressing, no 64-bit multiplies per load).
@@ -376,6 +352,42 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 #pragma unroll
     for (int s0 = 0; s0 < NSTAGE; ++s0)
         if (s0 < n_my) issue_tile(wave + s0 * NW, s0);
+    // (The first tiles are already on their way: the query's own loads, and in the
+    // append variant its normalisation, overlap with them.)
+    // Query group as the MFMA B operand (zero columns beyond the group). The
+    // load itself is unpredicated (padding lanes re-read the last head) so
+    // that it does not force a full wait on the first K/V tile.
+    {
+        const int hq = kvh * a.group + min(n16, a.group - 1);
+        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim;
+        const bool live = n16 < a.group;
+        if constexpr (APPEND) {
+            norm_rope_row(qp, a.norm_w, a.sin_row, a.cos_row, a.eps, kg, qb);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) qb[j] = *reinterpret_cast<const u32x4*>(qp + kg * 8 + j * 32);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qb[j] = live ? qb[j] : u32x4{0u, 0u, 0u, 0u};
+    }
+    // Fused append: the last tile of the last split holds the new token. Its K row
+    // (normalised + rotated here) and V row are used from registers and stored to
+    // the cache by the wave that owns that tile.
+    if constexpr (APPEND) {
+        if (holds_new_row) {
+            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_row, a.cos_row, a.eps, kg, k_fresh);
+            v_fresh = *reinterpret_cast<const u32x4*>(a.v_new + kvh * kHeadDim + n16 * 8);
+        }
+    }
+
+    // Pin the point where the query (and the fresh rows) must have arrived: here,
+    // before the loop. Left to itself the compiler waits for them at their first use
+    // inside the loop with vmcnt(0) on every trip -- it cannot see the LDS-DMA loads
+    // issued after them -- and that would also wait for every prefetched tile.
+    asm volatile("" ::"v"(qb[0]), "v"(qb[1]), "v"(qb[2]), "v"(qb[3]));
+    if constexpr (APPEND)
+        asm volatile("" ::"v"(k_fresh[0]), "v"(k_fresh[1]), "v"(k_fresh[2]), "v"(k_fresh[3]), "v"(v_fresh));
+
     int stage = 0;
     for (int i = 0; i < n_my; ++i) {
         TileRegs r;
