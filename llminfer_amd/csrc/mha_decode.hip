@@ -265,9 +265,13 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int kMerge4 = NW * 4 * G * kHeadDim * (int)sizeof(float) + kMergeTail;
     constexpr int kRows = kMerge4 <= 65536 ? 4 : 1;
     constexpr int kMergeBytes = NW * kRows * G * kHeadDim * (int)sizeof(float) + kMergeTail;
-    constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float);
-    constexpr int kSmemBytes = kRingBytes > kMergeBytes ? (kRingBytes > kCombineBytes ? kRingBytes : kCombineBytes)
-                                                        : (kMergeBytes > kCombineBytes ? kMergeBytes : kCombineBytes);
+    // Combine area (behind the merge area, so the merged (max, sum) pairs stay readable):
+    // weights [G][kMaxSplits], denominators [G], per-wave arrival flags [NW] and one
+    // 16-byte partial sum per thread.
+    constexpr int kCombineBase = (kMergeBytes + 15) & ~15;
+    constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float) + NW * 64 * 16;
+    constexpr int kTailBytes = kCombineBase + kCombineBytes;
+    constexpr int kSmemBytes = kRingBytes > kTailBytes ? kRingBytes : kTailBytes;
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * (NSTAGE * kStageBytes);
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
@@ -510,7 +514,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // The workgroup of the LAST split of this KV head merges the partials of its
     // query heads, so no second launch is needed. Every split publishes, per query
     // head, a record {epoch | max} {epoch | sum} after its partial outputs have been
-    // acknowledged; the last split's workgroup waits for all records. Workgroups are
+    // acknowledged; the last split's workgroup waits for all records but its own (it
+    // has its own pair in LDS and its own partials acknowledged). Workgroups are
     // dispatched in index order and the others never wait for anything, so whoever
     // it waits for is already running or done.
     // A record carries the epoch of the call that wrote it; anything else (an
@@ -521,7 +526,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     __syncthreads();
     const int S = a.num_splits;
     const unsigned long long tag = a.epoch & 0xffffffffull;
-    if (threadIdx.x < a.group) {
+    if (split != S - 1 && threadIdx.x < a.group) {
         const int h = threadIdx.x;
         unsigned long long* rec = a.records + ((int64_t)(kvh * a.group + h) * S + split) * 2;
         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h]);
@@ -531,13 +536,15 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     }
     if (split != S - 1) return;
 
-    __syncthreads();  // s_fin has been read: the merge area may be reused below
-    float* s_w = reinterpret_cast<float*>(smem);                                     // [G][kMaxSplits] weights
-    float* s_den = reinterpret_cast<float*>(smem + G * kMaxSplits * sizeof(float));  // [G] denominators
-    int* s_ok = reinterpret_cast<int*>(s_den + G);                                   // [NW] every record seen
+    float* s_w = reinterpret_cast<float*>(smem + kCombineBase);  // [G][kMaxSplits] weights
+    float* s_den = s_w + G * kMaxSplits;                         // [G] denominators
+    int* s_ok = reinterpret_cast<int*>(s_den + G);               // [NW] every record seen
+    f32x4* s_part = reinterpret_cast<f32x4*>(s_ok + NW);         // [NW * 64] per-thread partial sums
     bool wave_ok = true;
     // One wave per head: wait for the head's records, then M = max m_s, weights
     // e^(m_s - M), denominator sum l_s * weight -- all from the polled registers.
+    // This workgroup's own (max, sum) comes straight from LDS: its record would be
+    // the last one to become visible.
     for (int h = wave; h < a.group; h += NW) {
         unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         constexpr int kSlots = kMaxSplits / 64;
@@ -552,16 +559,19 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 const int sp = lane + 64 * j;
                 m_reg[j] = -INFINITY;
                 l_reg[j] = 0.0f;
-                if (sp < S) {
+                if (sp < S - 1) {
                     const unsigned long long r0 = __hip_atomic_load(rec + 2 * sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     const unsigned long long r1 = __hip_atomic_load(rec + 2 * sp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     ok = ok && (r0 & 0xffffffffull) == tag && (r1 & 0xffffffffull) == tag;
                     m_reg[j] = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
                     l_reg[j] = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
+                } else if (sp == S - 1) {
+                    m_reg[j] = s_fin[2 * h];
+                    l_reg[j] = s_fin[2 * h + 1];
                 }
             }
             if (__all(ok)) break;
-            __builtin_amdgcn_s_sleep(4);
+            __builtin_amdgcn_s_sleep(2);
         }
         wave_ok = wave_ok && __all(ok);
         float mx = -INFINITY;
@@ -577,8 +587,10 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 const float f = (m_reg[j] == -INFINITY) ? 0.0f : fast_exp2(m_reg[j] - mx);
                 s_w[h * kMaxSplits + sp] = f;
                 den += l_reg[j] * f;
-                __hip_atomic_store(rec + 2 * sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(rec + 2 * sp + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (sp < S - 1) {
+                    __hip_atomic_store(rec + 2 * sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(rec + 2 * sp + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
 #pragma unroll
@@ -590,28 +602,73 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     bool all_arrived = true;
 #pragma unroll
     for (int w = 0; w < NW; ++w) all_arrived = all_arrived && s_ok[w] != 0;
-    // Every other workgroup's partials were acknowledged before its records were
-    // written; read them with device-coherent loads.
-    auto coherent = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
-        const int h = idx >> 7;
-        const int d = idx & (kHeadDim - 1);
+
+    // Weighted sum of the partial outputs. Every other workgroup's partials were
+    // acknowledged before its records were written; they are read with device-coherent
+    // (L2-bypassing) 16-byte loads, a thread's loads all in flight at once, so that
+    // the time does not depend on how the split count divides. A thread owns four
+    // output columns of one head for every P-th split; the P partitions are added up
+    // through LDS.
+    constexpr int NT = NW * 64;
+    const int units = a.group * (kHeadDim / 4);
+    const int parts = units <= NT ? NT / units : 1;
+    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.ws, 0, (int)((int64_t)a.n_q * S * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
+    constexpr int kCoherent = 16;  // cache policy: sc1
+    for (int u0 = 0; u0 < units; u0 += NT) {
+        const int t = u0 + (int)threadIdx.x;
+        const int u = t % units;
+        const int part = units <= NT ? (int)threadIdx.x / units : 0;
+        const bool active = (units <= NT) ? part < parts : t < units;
+        const int h = u >> 5;
+        const int c4 = u & 31;
         const int hq = kvh * a.group + h;
-        const float* os = a.ws + (int64_t)hq * S * kHeadDim + d;
+        const uint32_t base = (uint32_t)(((int64_t)hq * S * kHeadDim + c4 * 4) * (int64_t)sizeof(float));
         const float* w = s_w + h * kMaxSplits;
-        float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
-        int sp = 0;
-        for (; sp + 4 <= S; sp += 4) {
-            acc0 += coherent(os + (int64_t)(sp + 0) * kHeadDim) * w[sp + 0];
-            acc1 += coherent(os + (int64_t)(sp + 1) * kHeadDim) * w[sp + 1];
-            acc2 += coherent(os + (int64_t)(sp + 2) * kHeadDim) * w[sp + 2];
-            acc3 += coherent(os + (int64_t)(sp + 3) * kHeadDim) * w[sp + 3];
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        // All of a batch's loads are issued before the first one is used; a short list
+        // of splits takes the small batch so that it does not pay for repeats.
+        auto gather = [&](auto batch) {
+            constexpr int kBatch = decltype(batch)::value;
+            for (int s0 = part; s0 < S; s0 += kBatch * parts) {
+                f32x4 v[kBatch];
+                float wv[kBatch];
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const int sp = s0 + j * parts;
+                    const int spc = min(sp, S - 1);  // in range; the weight below drops the repeat
+                    v[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                         ws_rsrc, base + (uint32_t)spc * (kHeadDim * 4u), 0, kCoherent));
+                    wv[j] = sp < S ? w[sp] : 0.0f;
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) acc += v[j] * wv[j];
+            }
+        };
+        if (active) {
+            if (S <= 8 * parts) gather(std::integral_constant<int, 8>{});
+            else gather(std::integral_constant<int, 16>{});
         }
-        for (; sp < S; ++sp) acc0 += coherent(os + (int64_t)sp * kHeadDim) * w[sp];
-        // A wait that ran out of patience poisons the output rather than returning a partial sum.
-        const float r = all_arrived ? ((acc0 + acc1) + (acc2 + acc3)) / s_den[h] : __builtin_nanf("");
-        a.out[(int64_t)hq * kHeadDim + d] = f32_to_bf16(r);
-        if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
+        if (units <= NT && parts > 1) {
+            s_part[threadIdx.x] = acc;
+            __syncthreads();
+            if (part == 0)
+                for (int pp = 1; pp < parts; ++pp) acc += s_part[pp * units + u];
+        }
+        if (active && part == 0) {
+            // A wait that ran out of patience poisons the output rather than returning a partial sum.
+            const float inv = all_arrived ? 1.0f / s_den[h] : __builtin_nanf("");
+            const f32x4 r = acc * inv;
+            uint16_t* op = a.out + (int64_t)hq * kHeadDim + c4 * 4;
+            const uint32_t lo = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
+            const uint32_t hi = (uint32_t)f32_to_bf16(r[2]) | ((uint32_t)f32_to_bf16(r[3]) << 16);
+            *reinterpret_cast<uint2*>(op) = make_uint2(lo, hi);
+            if (a.out_f32) {
+                float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
+#pragma unroll
+                for (int e = 0; e < 4; ++e) of[e] = r[e];
+            }
+        }
     }
 }
 
@@ -662,11 +719,14 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
 #ifndef LLMI_STAGES
 #define LLMI_STAGES 2
 #endif
+#ifndef LLMI_RING_LIMIT
+#define LLMI_RING_LIMIT 65536
+#endif
 
 template <int G, int NW>
 void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stream) {
-    // The LDS-DMA offset register addresses 64 KiB: NW * NSTAGE * 8 KiB must fit.
-    constexpr int kStages = (NW * LLMI_STAGES * 8192 <= 65536) ? LLMI_STAGES : 65536 / (NW * 8192);
+    // NW * NSTAGE * 8 KiB of ring must fit the LDS budget of one workgroup.
+    constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
     dim3 grid(ka.num_splits, n_kv);
     if (append) {
         if constexpr (NW <= 4) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true>), grid, dim3(NW * 64), 0, stream, ka);
