@@ -44,6 +44,8 @@ namespace llmi {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -88,6 +90,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Two floats rounded to nearest even into one dword of bf16 (lo = a, hi = b).
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
 
 // 16 bytes per lane from global memory straight into LDS, no VGPR round trip:
 // lane L's bytes land at lds_off + 16*L. `base` and `lds_off` are wave-uniform,
@@ -246,11 +255,11 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 
     float m_run = -INFINITY;  // running max, exp2 domain, per (head = n16)
     float l_run = 0.0f;       // running sum over this lane's rows
-    float o[G][8];
+    // Output accumulators, MFMA C layout of P^T V: o[j][r] belongs to head 4*kg + r and
+    // column 8*n16 + j, summed over all positions this wave has seen.
+    f32x4 o[8];
 #pragma unroll
-    for (int h = 0; h < G; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[h][e] = 0.0f;
+    for (int j = 0; j < 8; ++j) o[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     // Each wave streams its tiles through a private ring of NSTAGE LDS slots
     // (8 KiB each: 4 KiB of K rows, 4 KiB of V rows) filled by LDS-DMA loads,
@@ -260,11 +269,9 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // tile read the last valid row and are masked out of the softmax.
     constexpr int kStageBytes = 8192;
     constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
-    // Merge area: NW x kRows x G x 128 partial outputs + per-wave and merged (max, sum) pairs.
+    // Merge area: NW x G x 128 partial outputs + per-wave and merged (max, sum) pairs.
     constexpr int kMergeTail = (2 * NW * G + 2 * G) * (int)sizeof(float);
-    constexpr int kMerge4 = NW * 4 * G * kHeadDim * (int)sizeof(float) + kMergeTail;
-    constexpr int kRows = kMerge4 <= 65536 ? 4 : 1;
-    constexpr int kMergeBytes = NW * kRows * G * kHeadDim * (int)sizeof(float) + kMergeTail;
+    constexpr int kMergeBytes = NW * G * kHeadDim * (int)sizeof(float) + kMergeTail;
     // Combine area (behind the merge area, so the merged (max, sum) pairs stay readable):
     // weights [G][kMaxSplits], denominators [G], per-wave arrival flags [NW] and one
     // 16-byte partial sum per thread.
@@ -318,37 +325,46 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = fast_exp2(m_run - m_new);
         float p[4];
-        float psum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            p[i] = fast_exp2(s[i] - m_new);
-            psum += p[i];
-        }
+        for (int i = 0; i < 4; ++i) p[i] = fast_exp2(s[i] - m_new);
+        // The probabilities enter the second MFMA as a sum of two bf16 numbers
+        // (p = hi + lo, relative error 2^-17), so that the product keeps fp32-like accuracy.
+        const uint32_t p01 = pack_bf16(p[0], p[1]);
+        const uint32_t p23 = pack_bf16(p[2], p[3]);
+        const uint32_t q01 = pack_bf16(p[0] - bf16_lo(p01), p[1] - bf16_hi(p01));
+        const uint32_t q23 = pack_bf16(p[2] - bf16_lo(p23), p[3] - bf16_hi(p23));
+        const float psum = (p[0] + p[1]) + (p[2] + p[3]);
         l_run = l_run * alpha + psum;
         m_run = m_new;
 
-        // Rescale only when some head's max moved (wave-uniform test).
+        // Rescale only when some head's max moved (wave-uniform test). The factor of
+        // head 4*kg + r sits in lane 4*kg + r of this lane's 16-lane row.
         if (__any(alpha != 1.0f)) {
-            static_for<0, G>([&](auto h) {
-                const float ah = row_bcast<h.value>(alpha);
+            static_for<0, 4>([&](auto r) {
+                float ar;
+                if constexpr (G <= 4) ar = row_bcast<r.value>(alpha);  // only row kg = 0 holds heads
+                else ar = __shfl(alpha, (lane & 48) + 4 * kg + r.value);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[h.value][e] *= ah;
+                for (int j = 0; j < 8; ++j) o[j][r.value] *= ar;
             });
         }
+        // O^T += P^T V on the matrix cores: A = P^T (head x position: this lane's four
+        // probabilities are exactly its A fragment), B = V (position x column, column
+        // 8*n + j for output lane n: element j of each of the lane's four V rows).
+        const i16x4 pa = __builtin_bit_cast(i16x4, u32x2{p01, p23});
+        const i16x4 pb = __builtin_bit_cast(i16x4, u32x2{q01, q23});
+        i16x4 vb[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float vf[8];
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                vf[2 * w] = bf16_lo(r.v[i][w]);
-                vf[2 * w + 1] = bf16_hi(r.v[i][w]);
-            }
-            static_for<0, G>([&](auto h) {
-                const float ph = row_bcast<h.value>(p[i]);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[h.value][e] = __builtin_fmaf(ph, vf[e], o[h.value][e]);
-            });
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;  // high or low halves
+            const uint32_t b01 = __builtin_amdgcn_perm(r.v[1][j >> 1], r.v[0][j >> 1], sel);
+            const uint32_t b23 = __builtin_amdgcn_perm(r.v[3][j >> 1], r.v[2][j >> 1], sel);
+            vb[j] = __builtin_bit_cast(i16x4, u32x2{b01, b23});
         }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb[j], o[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pb, vb[j], o[j], 0, 0, 0);
     };
 
     // Wave w owns tiles w, w+NW, ...: NSTAGE of them are always in flight.
@@ -421,40 +437,28 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
     }
 
-    // ---- epilogue: fold the wave's four DPP rows and the workgroup's waves ----
-    // Each DPP row (kg) holds a partial sum over its own positions; all rows share
-    // the running max of a head, so rows add up plainly. When LDS has room the
-    // four rows are written side by side and summed by the merge below (no
-    // cross-lane traffic at all); otherwise they are folded with xor shuffles first.
+    // ---- epilogue: fold the workgroup's waves ----
+    // The outputs are already summed over a wave's positions; the denominators are
+    // per DPP row (kg) and share the running max of their head, so they add up plainly.
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
-    if constexpr (kRows == 1) {
-#pragma unroll
-        for (int h = 0; h < G; ++h)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float x = o[h][e];
-                x += __shfl_xor(x, 16);
-                x += __shfl_xor(x, 32);
-                o[h][e] = x;
-            }
-    }
 
     // The ring is drained (every tile issued was waited for): reuse its memory
     // once all waves are done with it.
     __syncthreads();
-    typedef float (*MergeO)[kRows][G][kHeadDim];
+    typedef float (*MergeO)[G][kHeadDim];
     typedef float (*MergeS)[G];
     MergeO s_o = reinterpret_cast<MergeO>(smem);
-    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * kRows * G * kHeadDim * sizeof(float));
+    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * G * kHeadDim * sizeof(float));
     MergeS s_l = s_m + NW;
     float* s_fin = reinterpret_cast<float*>(s_l + NW);  // [G][2]: merged (max, sum) per head
-    if (kRows == 4 || kg == 0) {
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            float* dst = &s_o[wave][kRows == 4 ? kg : 0][h][n16 * 8];
-            *reinterpret_cast<f32x4*>(dst) = f32x4{o[h][0], o[h][1], o[h][2], o[h][3]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[h][4], o[h][5], o[h][6], o[h][7]};
+    for (int r = 0; r < 4; ++r) {
+        const int h = 4 * kg + r;
+        if (h < G) {
+            float* dst = &s_o[wave][h][n16 * 8];
+            *reinterpret_cast<f32x4*>(dst) = f32x4{o[0][r], o[1][r], o[2][r], o[3][r]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[4][r], o[5][r], o[6][r], o[7][r]};
         }
     }
     if (kg == 0 && n16 < G) {
@@ -476,10 +480,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         for (int w = 0; w < NW; ++w) {
             const float mw = s_m[w][h];
             const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - mx);
-            float rows = s_o[w][0][h][d];
-#pragma unroll
-            for (int r = 1; r < kRows; ++r) rows += s_o[w][r][h][d];
-            acc += rows * f;
+            acc += s_o[w][h][d] * f;
             lsum += s_l[w][h] * f;
         }
         const int hq = kvh * a.group + h;
