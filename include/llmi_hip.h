@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define LLMI_HIP_ABI_VERSION 1
+#define LLMI_HIP_ABI_VERSION 2
 
 typedef enum llmi_status {
     LLMI_OK = 0,
@@ -93,6 +93,12 @@ typedef struct llmi_mha_args {
     int32_t num_splits;       /* 0 = auto; otherwise the KV split count of the split path */
     int32_t waves_per_group;  /* 0 = auto; 1,2,4,8 wavefronts per workgroup (tuning)     */
     void* stream;             /* hipStream_t, NULL = the null stream                     */
+    const int32_t* pos_device; /* optional, device int32: when non-NULL the kernels read the position
+                                 from here at run time, so one captured launch serves every token
+                                 up to `pos`, which then is the LARGEST position the launch may see
+                                 (it sizes the grid; larger values read from the device are clamped
+                                 to it). The reference bakes pos into the launch (mha.cpp:55,60-66).
+                                 Not available with LLMI_PATH_SPLIT.                       */
 } llmi_mha_args;
 
 typedef struct llmi_mha_plan {

@@ -30,7 +30,7 @@ class MhaArgs(ctypes.Structure):
         ("layer_id", c_i32), ("pos", c_i32), ("kv_dim", c_i32), ("kv_mul", c_i32),
         ("head_num", c_i32), ("head_dim", c_i32), ("max_seq_len", c_i32), ("kv_layout", c_i32),
         ("force_path", c_i32), ("num_splits", c_i32), ("waves_per_group", c_i32),
-        ("stream", c_void_p),
+        ("stream", c_void_p), ("pos_device", c_void_p),
     ]
 
 

@@ -82,6 +82,7 @@ static int validate_mha(const llmi_mha_args* a) {
         return LLMI_ERR_ALIGNMENT;                                                  // mha_kernel.cu:495-498
     if (a->workspace && !aligned16(a->workspace)) return LLMI_ERR_ALIGNMENT;
     if (a->output_f32 && (reinterpret_cast<uintptr_t>(a->output_f32) & 3u)) return LLMI_ERR_ALIGNMENT;
+    if (a->pos_device && (reinterpret_cast<uintptr_t>(a->pos_device) & 3u)) return LLMI_ERR_ALIGNMENT;
     if (a->force_path < LLMI_PATH_AUTO || a->force_path > LLMI_PATH_SPLIT_FUSED) return LLMI_ERR_INVALID_ARG;
     if (a->num_splits < 0 || a->num_splits > kMaxSplits) return LLMI_ERR_INVALID_ARG;
     const int w = a->waves_per_group;
@@ -110,6 +111,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
         else path = seq_len <= kSinglePassMaxLen ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT_FUSED;
         if (path == LLMI_PATH_SPLIT) path = LLMI_PATH_SPLIT_FUSED;
     }
+    // The separate combine kernel takes its split count from the launch, not from the device.
+    if (a->pos_device && path == LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
 
     int num_splits = 1, tiles_per_split = tiles, waves;
     if (path != LLMI_PATH_SINGLE_PASS) {

@@ -142,6 +142,7 @@ struct KernelArgs {
     float* out_f32;       // optional
     unsigned long long* records;   // [n_q][num_splits][2] arrival records of the fused combine, or nullptr
     unsigned long long epoch;      // tag of this call, 48 bits
+    const int32_t* pos_dev;        // optional: position read at run time (seq_len then is its upper bound + 1)
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
@@ -156,11 +157,9 @@ struct KernelArgs {
     const uint16_t* k_new;   // [n_kv][128] raw
     const uint16_t* v_new;   // [n_kv][128]
     const uint16_t* norm_w;  // [2][128]: q_norm, k_norm
-    const float* sin_row;    // [64] of this position
-    const float* cos_row;
-    uint16_t* k_slot;        // cache address of (layer, seq_len-1, kv_head 0)
-    uint16_t* v_slot;
-    int64_t slot_head_stride;
+    const float* sin_cache;  // [max_seq_len][64]
+    const float* cos_cache;
+    int64_t slot_head_stride;  // elements between KV heads inside a slot
     float eps;
 };
 
@@ -223,7 +222,7 @@ __device__ __forceinline__ void norm_rope_row(const uint16_t* row, const uint16_
     }
 }
 
-template <int G, int NW, int NSTAGE, bool APPEND>
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN>
 __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
@@ -232,15 +231,28 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
 
-    const int begin = split * a.rows_per_split;
-    const int nrows = min(a.rows_per_split, a.seq_len - begin);  // > 0: the host never makes empty splits
+    // Static launch: the host never makes empty splits. With a position read from
+    // device memory the grid was sized for the largest position; the same rule as the
+    // host's (equal tile counts, no empty split in the middle) is applied here, and the
+    // workgroups beyond the last active split leave at once.
+    int seq_len = a.seq_len, rows_per_split = a.rows_per_split, n_active = a.num_splits;
+    if constexpr (DYN) {
+        seq_len = max(0, min(*a.pos_dev, a.seq_len - 1)) + 1;
+        const int tiles = (seq_len + kTile - 1) / kTile;
+        const int tps = (tiles + a.num_splits - 1) / a.num_splits;
+        rows_per_split = tps * kTile;
+        n_active = (tiles + tps - 1) / tps;
+        if (split >= n_active) return;
+    }
+    const int begin = split * rows_per_split;
+    const int nrows = min(rows_per_split, seq_len - begin);  // > 0
     const int ntiles = (nrows + kTile - 1) / kTile;
 
     // Filled in below, once the first tiles are on their way.
     u32x4 qb[4];                       // query group, MFMA B operand
     u32x4 k_fresh[4] = {};             // append variant: the new token's K row (operand layout) ...
     u32x4 v_fresh = {0u, 0u, 0u, 0u};  // ... and V row chunk
-    const bool holds_new_row = APPEND && split == a.num_splits - 1;
+    const bool holds_new_row = APPEND && split == n_active - 1;
 
     // Wave-uniform 64-bit bases of this split; lanes add 32-bit byte offsets
     // (scalar-base + vector-offset addressing, no 64-bit multiplies per load).
@@ -382,7 +394,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         const uint16_t* qp = a.q + (int64_t)hq * kHeadDim;
         const bool live = n16 < a.group;
         if constexpr (APPEND) {
-            norm_rope_row(qp, a.norm_w, a.sin_row, a.cos_row, a.eps, kg, qb);
+            norm_rope_row(qp, a.norm_w, a.sin_cache + (int64_t)(seq_len - 1) * 64, a.cos_cache + (int64_t)(seq_len - 1) * 64,
+                          a.eps, kg, qb);
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) qb[j] = *reinterpret_cast<const u32x4*>(qp + kg * 8 + j * 32);
@@ -395,7 +408,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // the cache by the wave that owns that tile.
     if constexpr (APPEND) {
         if (holds_new_row) {
-            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_row, a.cos_row, a.eps, kg, k_fresh);
+            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_cache + (int64_t)(seq_len - 1) * 64,
+                          a.cos_cache + (int64_t)(seq_len - 1) * 64, a.eps, kg, k_fresh);
             v_fresh = *reinterpret_cast<const u32x4*>(a.v_new + kvh * kHeadDim + n16 * 8);
         }
     }
@@ -425,11 +439,13 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) r.v[q4] = 4 * kg + q4 >= fresh ? v_fresh : r.v[q4];
                 if (n16 == 0) {
-                    uint16_t* kd = a.k_slot + kvh * a.slot_head_stride;
+                    uint16_t* kd = const_cast<uint16_t*>(a.k) + (int64_t)(seq_len - 1) * a.row_stride + kvh * a.slot_head_stride;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = k_fresh[j];
                 }
-                if (kg == 0) *reinterpret_cast<u32x4*>(a.v_slot + kvh * a.slot_head_stride + n16 * 8) = v_fresh;
+                if (kg == 0)
+                    *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + (int64_t)(seq_len - 1) * a.row_stride +
+                                              kvh * a.slot_head_stride + n16 * 8) = v_fresh;
             }
         }
         if (i + NSTAGE < n_my) issue_tile(wave + (i + NSTAGE) * NW, stage);
@@ -467,7 +483,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     }
     __syncthreads();
 
-    const bool fused = a.records != nullptr && a.num_splits > 1;
+    const bool fused = a.records != nullptr && n_active > 1;
     const int n_out = a.group * kHeadDim;
     for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
         const int h = idx >> 7;
@@ -484,7 +500,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
             lsum += s_l[w][h] * f;
         }
         const int hq = kvh * a.group + h;
-        if (a.num_splits == 1) {
+        if (n_active == 1) {
             const float r = acc / lsum;
             a.out[(int64_t)hq * kHeadDim + d] = f32_to_bf16(r);
             if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
@@ -525,9 +541,10 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // graph replay of this very call (same epoch) starts clean.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
     __syncthreads();
-    const int S = a.num_splits;
+    const int S = a.num_splits;  // layout stride of partials and records
+    const int SA = n_active;     // splits that hold positions
     const unsigned long long tag = a.epoch & 0xffffffffull;
-    if (split != S - 1 && threadIdx.x < a.group) {
+    if (split != SA - 1 && threadIdx.x < a.group) {
         const int h = threadIdx.x;
         unsigned long long* rec = a.records + ((int64_t)(kvh * a.group + h) * S + split) * 2;
         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h]);
@@ -535,7 +552,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(rec + 1, tag | (l_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (split != S - 1) return;
+    if (split != SA - 1) return;
 
     float* s_w = reinterpret_cast<float*>(smem + kCombineBase);  // [G][kMaxSplits] weights
     float* s_den = s_w + G * kMaxSplits;                         // [G] denominators
@@ -560,13 +577,13 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 const int sp = lane + 64 * j;
                 m_reg[j] = -INFINITY;
                 l_reg[j] = 0.0f;
-                if (sp < S - 1) {
+                if (sp < SA - 1) {
                     const unsigned long long r0 = __hip_atomic_load(rec + 2 * sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     const unsigned long long r1 = __hip_atomic_load(rec + 2 * sp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     ok = ok && (r0 & 0xffffffffull) == tag && (r1 & 0xffffffffull) == tag;
                     m_reg[j] = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
                     l_reg[j] = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
-                } else if (sp == S - 1) {
+                } else if (sp == SA - 1) {
                     m_reg[j] = s_fin[2 * h];
                     l_reg[j] = s_fin[2 * h + 1];
                 }
@@ -584,11 +601,11 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) {
             const int sp = lane + 64 * j;
-            if (sp < S) {
+            if (sp < SA) {
                 const float f = (m_reg[j] == -INFINITY) ? 0.0f : fast_exp2(m_reg[j] - mx);
                 s_w[h * kMaxSplits + sp] = f;
                 den += l_reg[j] * f;
-                if (sp < S - 1) {
+                if (sp < SA - 1) {
                     __hip_atomic_store(rec + 2 * sp, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(rec + 2 * sp + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
@@ -631,23 +648,23 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         // of splits takes the small batch so that it does not pay for repeats.
         auto gather = [&](auto batch) {
             constexpr int kBatch = decltype(batch)::value;
-            for (int s0 = part; s0 < S; s0 += kBatch * parts) {
+            for (int s0 = part; s0 < SA; s0 += kBatch * parts) {
                 f32x4 v[kBatch];
                 float wv[kBatch];
 #pragma unroll
                 for (int j = 0; j < kBatch; ++j) {
                     const int sp = s0 + j * parts;
-                    const int spc = min(sp, S - 1);  // in range; the weight below drops the repeat
+                    const int spc = min(sp, SA - 1);  // in range; the weight below drops the repeat
                     v[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
                                                          ws_rsrc, base + (uint32_t)spc * (kHeadDim * 4u), 0, kCoherent));
-                    wv[j] = sp < S ? w[sp] : 0.0f;
+                    wv[j] = sp < SA ? w[sp] : 0.0f;
                 }
 #pragma unroll
                 for (int j = 0; j < kBatch; ++j) acc += v[j] * wv[j];
             }
         };
         if (active) {
-            if (S <= 8 * parts) gather(std::integral_constant<int, 8>{});
+            if (SA <= 8 * parts) gather(std::integral_constant<int, 8>{});
             else gather(std::integral_constant<int, 16>{});
         }
         if (units <= NT && parts > 1) {
@@ -729,10 +746,15 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
     // NW * NSTAGE * 8 KiB of ring must fit the LDS budget of one workgroup.
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
     dim3 grid(ka.num_splits, n_kv);
+    const bool dyn = ka.pos_dev != nullptr;  // position read at run time: its own instantiation, the static one pays nothing
     if (append) {
-        if constexpr (NW <= 4) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true>), grid, dim3(NW * 64), 0, stream, ka);
+        if constexpr (NW <= 4) {
+            if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+            else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
+        }
     } else {
-        hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false>), grid, dim3(NW * 64), 0, stream, ka);
+        if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false>), grid, dim3(NW * 64), 0, stream, ka);
     }
 }
 
@@ -765,6 +787,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
     ka.out_f32 = args.output_f32;
     ka.records = nullptr;
     ka.epoch = 0;
+    ka.pos_dev = args.pos_device;
     if (plan.path == LLMI_PATH_SPLIT_FUSED) {
         // Arrival records sit behind the partial outputs in the workspace.
         const size_t partial_bytes = (size_t)args.head_num * plan.num_splits * args.head_dim * sizeof(float);
@@ -772,15 +795,12 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
                                                            ((partial_bytes + 15) & ~(size_t)15));
         ka.epoch = next_epoch();
     }
-    int64_t slot_off;
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
         ka.row_stride = args.kv_dim;
         ka.head_stride = args.head_dim;
-        slot_off = (int64_t)args.pos * args.kv_dim;
     } else {
         ka.row_stride = args.head_dim;
         ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
-        slot_off = (int64_t)args.pos * args.head_dim;
     }
     ka.seq_len = args.pos + 1;
     ka.group = args.kv_mul;
@@ -792,10 +812,8 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         ka.k_new = static_cast<const uint16_t*>(append->key_new);
         ka.v_new = static_cast<const uint16_t*>(append->value_new);
         ka.norm_w = static_cast<const uint16_t*>(append->norm_weight);
-        ka.sin_row = append->sin_cache + (int64_t)args.pos * (args.head_dim / 2);
-        ka.cos_row = append->cos_cache + (int64_t)args.pos * (args.head_dim / 2);
-        ka.k_slot = const_cast<uint16_t*>(ka.k) + slot_off;
-        ka.v_slot = const_cast<uint16_t*>(ka.v) + slot_off;
+        ka.sin_cache = append->sin_cache;
+        ka.cos_cache = append->cos_cache;
         ka.slot_head_stride = ka.head_stride;
         ka.eps = append->eps;
     }

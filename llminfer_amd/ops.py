@@ -36,7 +36,7 @@ def workspace_bytes(head_num, head_dim, max_seq_len):
 
 def make_mha_args(query, key_cache, value_cache, output, workspace, *, layer_id, pos, kv_dim, kv_mul,
                   head_num, head_dim, max_seq_len, kv_layout=B.KV_LAYOUT_POS_MAJOR, force_path=B.PATH_AUTO,
-                  num_splits=0, waves_per_group=0, output_f32=None, stream=None):
+                  num_splits=0, waves_per_group=0, output_f32=None, stream=None, pos_device=None):
     """Fills an llmi_mha_args from torch tensors (or raw integer addresses)."""
     def addr(x):
         return x if (x is None or isinstance(x, int)) else x.data_ptr()
@@ -58,6 +58,7 @@ def make_mha_args(query, key_cache, value_cache, output, workspace, *, layer_id,
     a.head_num, a.head_dim, a.max_seq_len = head_num, head_dim, max_seq_len
     a.kv_layout, a.force_path, a.num_splits, a.waves_per_group = kv_layout, force_path, num_splits, waves_per_group
     a.stream = stream
+    a.pos_device = addr(pos_device)
     return a
 
 

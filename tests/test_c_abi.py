@@ -31,7 +31,7 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(lib, name), "libllmi_hip.so does not export " + name
         assert name in B.SYMBOLS, "the ctypes binding does not declare " + name
     assert set(B.SYMBOLS) == set(names)
-    assert lib.llmi_hip_abi_version() == 1
+    assert lib.llmi_hip_abi_version() == 2
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -141,6 +141,17 @@ def test_plan_honours_requests_and_clamps_to_the_workspace():
     assert rc == 0 and p.group_pad == 16 and p.waves_per_group <= 4
     rc, _ = plan(good_args(kv_mul=16, head_num=128, waves_per_group=8))
     assert rc == B.STATUS["INVALID_ARG"]
+
+
+def test_plan_with_a_device_position():
+    """pos_device: pos is the largest position the launch serves; the separate combine kernel cannot follow
+    a position it does not read, and the pointer must be int32-aligned."""
+    rc, p = plan(good_args(pos_device=0x1000))
+    assert rc == 0 and p.path == B.PATH_SPLIT_FUSED
+    rc, _ = plan(good_args(pos_device=0x1000, force_path=B.PATH_SPLIT, num_splits=8))
+    assert rc == B.STATUS["INVALID_ARG"]
+    rc, _ = plan(good_args(pos_device=0x1002))
+    assert rc == B.STATUS["ALIGNMENT"]
 
 
 def test_workspace_bytes():
