@@ -154,7 +154,13 @@ def run_stack(args, ctx):
         up(host.llmi_host_stack_ptr(st, 5, l),
            synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * HEAD_DIM)).astype(np.float32)))
     ok(host.llmi_host_stack_run(st, pos, args.stack_mode))
-    ok(host.llmi_host_stack_capture(st, pos, args.stack_mode))
+    if args.stack_follow_pos:
+        host.llmi_host_stack_capture_following.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+        host.llmi_host_stack_set_pos.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+        ok(host.llmi_host_stack_set_pos(st, pos))
+        ok(host.llmi_host_stack_capture_following(st, msl - 1, args.stack_mode))
+    else:
+        ok(host.llmi_host_stack_capture(st, pos, args.stack_mode))
     ms = ctypes.c_float()
     ok(host.llmi_host_stack_replay(st, max(1, args.warmup), ctypes.byref(ms)))
     ok(host.llmi_host_stack_replay(st, args.steps, ctypes.byref(ms)))
@@ -169,7 +175,8 @@ def run_stack(args, ctx):
         "config": {"workload": "%d layers x (fused QK-Norm + RoPE + K/V append, GQA decode attention), %d Q / 8 KV "
                                "heads, ctx %d + 1 new token, one HIP graph per token, %s layout, %s"
                                % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major",
-                                  "one launch per layer" if args.stack_mode == 2 else "two launches per layer")},
+                                  "one launch per layer" if args.stack_mode == 2 else "two launches per layer")
+                            + (", position read from device memory" if args.stack_follow_pos else "")},
         "us_per_layer": round(us_token / layers, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
@@ -189,6 +196,8 @@ def main():
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
                     help="instead of the sweep: LAYERS layers of (QK-Norm + RoPE + append, attention) at --ctx (one "
                          "value) + 1 new token, captured into one HIP graph; reports us per token")
+    ap.add_argument("--stack-follow-pos", action="store_true",
+                    help="with --stack: capture once for every position (kernels read it from device memory)")
     ap.add_argument("--stack-mode", type=int, default=2,
                     help="with --stack: 2 = norm/rope/append fused into the attention launch (default), "
                          "1 = separate kernel before attention (the reference's sequence)")

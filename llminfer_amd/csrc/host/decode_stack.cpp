@@ -24,6 +24,8 @@ DecodeStack::DecodeStack(const AttentionConfig& config) : config_(config) {
     raw_v_ = tensor::Tensor(DataType::DataTypeBf16, L, config.kv_dim(), true, alloc);
     norm_w_ = tensor::Tensor(DataType::DataTypeBf16, L, 2 * config.head_dim, true, alloc);
     outputs_ = tensor::Tensor(DataType::DataTypeBf16, L, config.dim(), true, alloc);
+    pos_dev_ = tensor::Tensor(DataType::DataTypeInt32, 4, true, alloc);
+    LLMI_CHECK(!pos_dev_.is_empty());
     LLMI_CHECK(!raw_q_.is_empty() && !raw_k_.is_empty() && !raw_v_.is_empty() && !norm_w_.is_empty() && !outputs_.is_empty());
 }
 
@@ -39,8 +41,9 @@ void DecodeStack::build_sincos() {
     synchronize();
 }
 
-void DecodeStack::enqueue(int32_t pos, int32_t mode) {
+void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
     const bool with_qk_norm_rope = mode == kSeparateQkNormRope;
+    LLMI_CHECK(!(follow_device_pos && with_qk_norm_rope));
     const AttentionConfig& c = config_;
     tensor::Tensor& kc = buffers_->get_buffer(ModelBufferType::KeyCache);
     tensor::Tensor& vc = buffers_->get_buffer(ModelBufferType::ValueCache);
@@ -92,6 +95,7 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode) {
         m.num_splits = o.num_splits;
         m.waves_per_group = o.waves_per_group;
         m.stream = stream();
+        m.pos_device = follow_device_pos ? pos_dev_.ptr<int32_t>() : nullptr;
         int rc;
         if (mode == kFusedAppend) {
             llmi_mha_append_args f{};
@@ -111,7 +115,14 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode) {
     }
 }
 
-void DecodeStack::capture(int32_t pos, int32_t mode) {
+void DecodeStack::set_position(int32_t pos) {
+    // Synchronous small copy: the word is in place before anything enqueued afterwards runs.
+    synchronize();
+    const int rc = llmi_hip_memcpy(pos_dev_.ptr<int32_t>(), &pos, sizeof(pos), 1, nullptr, 1);
+    if (rc != LLMI_OK) LLMI_FATAL("set_position: " << llmi_hip_strerror(rc));
+}
+
+void DecodeStack::capture(int32_t pos, int32_t mode, bool follow_device_pos) {
     if (graph_exec_) {
         HIP_OK(hipGraphExecDestroy(graph_exec_));
         graph_exec_ = nullptr;
@@ -122,7 +133,7 @@ void DecodeStack::capture(int32_t pos, int32_t mode) {
     }
     HIP_OK(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
     try {
-        enqueue(pos, mode);
+        enqueue(pos, mode, follow_device_pos);
     } catch (...) {
         hipGraph_t dead = nullptr;
         (void)hipStreamEndCapture(stream(), &dead);

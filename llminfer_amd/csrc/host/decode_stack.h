@@ -37,9 +37,14 @@ public:
     // followed by attention (1, the reference's sequence), or both fused into one launch (2).
     enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2 };
     // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
-    void enqueue(int32_t pos, int32_t mode);
-    // Captures enqueue(pos, mode) into a graph (replacing an earlier one).
-    void capture(int32_t pos, int32_t mode);
+    // `follow_device_pos`: the kernels read the position from the stack's device word (set_position)
+    // and `pos` is the largest position they may see; modes 0 and 2 only (the separate QK-Norm/RoPE
+    // launch takes its position from the host).
+    void enqueue(int32_t pos, int32_t mode, bool follow_device_pos = false);
+    // Captures enqueue(pos, mode, follow_device_pos) into a graph (replacing an earlier one).
+    void capture(int32_t pos, int32_t mode, bool follow_device_pos = false);
+    // Writes the position word the kernels follow (ordered on the stack's stream).
+    void set_position(int32_t pos);
     // Replays the captured graph `times` times; returns the elapsed milliseconds (HIP events on the stream).
     float replay(int32_t times);
     void synchronize();
@@ -48,7 +53,7 @@ private:
     AttentionConfig config_;
     std::shared_ptr<kernel::HipConfig> hip_config_;
     std::unique_ptr<AttentionBuffers> buffers_;
-    tensor::Tensor raw_q_, raw_k_, raw_v_, norm_w_, outputs_;
+    tensor::Tensor raw_q_, raw_k_, raw_v_, norm_w_, outputs_, pos_dev_;
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
 };

@@ -83,6 +83,14 @@ int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_nor
     return guarded([&] { s->impl->capture(pos, with_qk_norm_rope); });
 }
 
+int llmi_host_stack_capture_following(llmi_host_stack* s, int32_t max_pos, int32_t mode) {
+    return guarded([&] { s->impl->capture(max_pos, mode, true); });
+}
+
+int llmi_host_stack_set_pos(llmi_host_stack* s, int32_t pos) {
+    return guarded([&] { s->impl->set_position(pos); });
+}
+
 int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms) {
     return guarded([&] {
         const float ms = s->impl->replay(times);

@@ -26,6 +26,10 @@ int llmi_host_stack_build_sincos(llmi_host_stack* s);
 int llmi_host_stack_run(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);      /* eager + synchronise */
 int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);
 int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms);
+/* Captures the stack for every position up to max_pos: the kernels read the position from a device word
+ * (llmi_mha_args.pos_device) that llmi_host_stack_set_pos writes between replays. mode 0 or 2. */
+int llmi_host_stack_capture_following(llmi_host_stack* s, int32_t max_pos, int32_t mode);
+int llmi_host_stack_set_pos(llmi_host_stack* s, int32_t pos);
 /* Process-wide tuning overrides of the HIP attention arm (0 = automatic). */
 void llmi_host_set_mha_options(int32_t force_path, int32_t num_splits, int32_t waves_per_group);
 

@@ -319,6 +319,55 @@ def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout):
         H.L.llmi_host_stack_destroy(stack)
 
 
+def test_decode_stack_graph_follows_the_device_position(oracle, dev):
+    """One captured 3-layer stack (norm/rope/append fused into attention) decodes four successive tokens:
+    only the raw inputs and the position word change between replays."""
+    H = HostLib()
+    H.L.llmi_host_stack_capture_following.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
+    H.L.llmi_host_stack_set_pos.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+    layers, ctx, n_q, n_kv, d, tokens, layout = 3, 270, 32, 8, 128, 4, B.KV_LAYOUT_HEAD_MAJOR
+    msl, kv_dim = ctx + tokens, n_kv * d
+    stack = H.L.llmi_host_stack_create(layers, msl, n_q, n_kv, layout)
+    assert stack, H.L.llmi_host_last_error().decode()
+    try:
+        H.ok(H.L.llmi_host_stack_build_sincos(stack))
+        rng = np.random.RandomState(14)
+        k_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        v_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        ws = []
+        for l in range(layers):
+            c = synth.make_case(700 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+            k_all[l], v_all[l] = c["k"][0], c["v"][0]
+            w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+            ws.append(w)
+            _upload(H.L.llmi_host_stack_ptr(stack, 5, l), w)
+        _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), synth.to_head_major(k_all, n_kv))
+        _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), synth.to_head_major(v_all, n_kv))
+        sin_o, cos_o = oracle.sincos_table(d, msl)
+        H.ok(H.L.llmi_host_stack_set_pos(stack, ctx))
+        H.ok(H.L.llmi_host_stack_capture_following(stack, msl - 1, 2))
+        ms = ctypes.c_float()
+        for pos in range(ctx, ctx + tokens):
+            refs = []
+            for l in range(layers):
+                qr = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+                kr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+                vr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+                for which, arr in ((2, qr), (3, kr), (4, vr)):
+                    _upload(H.L.llmi_host_stack_ptr(stack, which, l), arr)
+                k_all[l, pos] = oracle.qk_norm_rope(kr, ws[l][d:], sin_o[pos], cos_o[pos]).reshape(-1)
+                v_all[l, pos] = vr.reshape(-1)
+                qn = oracle.qk_norm_rope(qr, ws[l][:d], sin_o[pos], cos_o[pos]).reshape(-1)
+                refs.append(oracle.mha_cpu(qn, k_all[l:l + 1], v_all[l:l + 1], 0, pos, kv_dim, n_q // n_kv, n_q, d, msl))
+            H.ok(H.L.llmi_host_stack_set_pos(stack, pos))
+            H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
+            for l in range(layers):
+                got = _download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16)
+                assert_parity(synth.bf16_bits_to_f32(got), refs[l], "token at %d, layer %d" % (pos, l))
+    finally:
+        H.L.llmi_host_stack_destroy(stack)
+
+
 def test_mha_op_forward_through_registry_hook(oracle, dev):
     """op::MultiHeadAttention::forward (C++ op layer -> registry -> HIP arm) on borrowed device tensors."""
     H = HostLib()
