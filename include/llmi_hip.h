@@ -227,6 +227,47 @@ int llmi_hip_memcpy(void* dst, const void* src, size_t bytes, int32_t kind, void
                     int32_t need_sync);
 int llmi_hip_memset_zero(void* ptr, size_t bytes, void* stream, int32_t need_sync);
 
+/* ---- the GEMVs either side of the attention -------------------------------- */
+/* Weights are bf16 [n][k] row-major, the input is bf16 [k], accumulation is fp32.
+ * k % 8 == 0; input, weight and outputs 16-byte aligned (matmul_kernel.cu:123-128). */
+enum {
+    LLMI_GEMV_OUT_BF16 = 0, /* output bf16 [n]                       gemv_kernel_cu, lm_head = false  */
+    LLMI_GEMV_OUT_F32 = 1,  /* output fp32 [n]                       gemv_kernel_cu, lm_head = true   */
+    LLMI_GEMV_ADD_BF16 = 2  /* output bf16 [n] += W x, rounded once  fused_gemv_add_kernel_cu         */
+};
+
+typedef struct llmi_gemv_args {
+    const void* input;   /* device bf16 [k]                                        */
+    const void* weight;  /* device bf16 [n][k]                                     */
+    void* output;        /* device [n], see the mode                               */
+    int32_t n;
+    int32_t k;
+    int32_t mode;        /* LLMI_GEMV_*                                            */
+    void* stream;        /* hipStream_t                                            */
+} llmi_gemv_args;
+
+/* Replaces gemv_kernel_cu (code/source/op/kernel/cuda/matmul_kernel.cu:100-141) and
+ * fused_gemv_add_kernel_cu (:174-208): one launch, allocates nothing, capturable. */
+int llmi_hip_gemv(const llmi_gemv_args* args);
+
+typedef struct llmi_qkv_gemv_args {
+    const void* input;   /* device bf16 [k]: the normalised hidden state            */
+    const void* weight;  /* device bf16 [dim + 2*kv_dim][k]: wq, wk, wv stacked      */
+    void* query;         /* device bf16 [dim]                                        */
+    void* key;           /* device bf16 [kv_dim]                                     */
+    void* value;         /* device bf16 [kv_dim]                                     */
+    int32_t dim;
+    int32_t kv_dim;
+    int32_t k;
+    void* stream;
+} llmi_qkv_gemv_args;
+
+/* Replaces fused_qkv_gemv_kernel_cu (matmul_kernel.cu:248-298). The reference points `key` and `value` at
+ * the cache row of the position (model.cpp:90-107); here they are the raw rows that
+ * llmi_hip_mha_decode_append (or llmi_hip_qk_norm_rope_append) normalises, rotates and files in the cache
+ * of either layout, so the GEMV needs no knowledge of the cache. */
+int llmi_hip_qkv_gemv(const llmi_qkv_gemv_args* args);
+
 /* ---- misc ---------------------------------------------------------------- */
 int llmi_hip_abi_version(void);
 const char* llmi_hip_strerror(int status);

@@ -41,6 +41,23 @@ class MhaAppendArgs(ctypes.Structure):
     ]
 
 
+class GemvArgs(ctypes.Structure):
+    _fields_ = [
+        ("input", c_void_p), ("weight", c_void_p), ("output", c_void_p),
+        ("n", c_i32), ("k", c_i32), ("mode", c_i32), ("stream", c_void_p),
+    ]
+
+
+class QkvGemvArgs(ctypes.Structure):
+    _fields_ = [
+        ("input", c_void_p), ("weight", c_void_p), ("query", c_void_p), ("key", c_void_p), ("value", c_void_p),
+        ("dim", c_i32), ("kv_dim", c_i32), ("k", c_i32), ("stream", c_void_p),
+    ]
+
+
+GEMV_OUT_BF16, GEMV_OUT_F32, GEMV_ADD_BF16 = 0, 1, 2
+
+
 class MhaPlan(ctypes.Structure):
     _fields_ = [
         ("path", c_i32), ("num_splits", c_i32), ("rows_per_split", c_i32),
@@ -78,6 +95,8 @@ SYMBOLS = {
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),
     "llmi_hip_sincos_table": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_void_p]),
     "llmi_hip_kv_restride": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p]),
+    "llmi_hip_gemv": (ctypes.c_int, [ctypes.POINTER(GemvArgs)]),
+    "llmi_hip_qkv_gemv": (ctypes.c_int, [ctypes.POINTER(QkvGemvArgs)]),
     "llmi_pool_create": (c_void_p, [BACKING_ALLOC_FN, BACKING_FREE_FN, c_void_p]),
     "llmi_pool_destroy": (None, [c_void_p]),
     "llmi_pool_alloc": (c_void_p, [c_void_p, c_size_t]),

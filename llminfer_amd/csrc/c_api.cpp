@@ -2,6 +2,7 @@
 // the hipMalloc-backed default pool and the copy helpers. The kernels live in
 // mha_decode.hip and qk_norm_rope.hip.
 
+#include <cstdint>
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -328,6 +329,32 @@ int llmi_hip_memset_zero(void* ptr, size_t bytes, void* stream, int32_t need_syn
     if (err != hipSuccess) return record_hip_error(err, "hipMemset");
     if (need_sync) return record_hip_error(hipDeviceSynchronize(), "hipDeviceSynchronize");
     return LLMI_OK;
+}
+
+int llmi_hip_gemv(const llmi_gemv_args* a) {
+    if (!a) return LLMI_ERR_NULL_POINTER;
+    if (!a->input || !a->weight || !a->output) return LLMI_ERR_NULL_POINTER;
+    if (a->n <= 0 || a->k <= 0 || a->k % 8 != 0) return LLMI_ERR_INVALID_ARG;  // matmul_kernel.cu:128
+    if (a->mode != LLMI_GEMV_OUT_BF16 && a->mode != LLMI_GEMV_OUT_F32 && a->mode != LLMI_GEMV_ADD_BF16)
+        return LLMI_ERR_INVALID_ARG;
+    if (!aligned16(a->input) || !aligned16(a->weight) || !aligned16(a->output)) return LLMI_ERR_ALIGNMENT;  // :123-124
+    void* const out[3] = {a->output, a->output, a->output};
+    const int32_t seg_end[3] = {a->n, a->n, a->n};
+    return launch_gemv(a->input, a->weight, out, seg_end, a->n, a->k, a->mode, static_cast<hipStream_t>(a->stream));
+}
+
+int llmi_hip_qkv_gemv(const llmi_qkv_gemv_args* a) {
+    if (!a) return LLMI_ERR_NULL_POINTER;
+    if (!a->input || !a->weight || !a->query || !a->key || !a->value) return LLMI_ERR_NULL_POINTER;
+    if (a->dim <= 0 || a->kv_dim <= 0 || a->k <= 0 || a->k % 8 != 0) return LLMI_ERR_INVALID_ARG;  // :290-292
+    if ((int64_t)a->dim + 2 * (int64_t)a->kv_dim > INT32_MAX) return LLMI_ERR_INVALID_ARG;
+    const void* ptrs[] = {a->input, a->weight, a->query, a->key, a->value};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
+    void* const out[3] = {a->query, a->key, a->value};
+    const int32_t seg_end[3] = {a->dim, a->dim + a->kv_dim, a->dim + 2 * a->kv_dim};
+    return launch_gemv(a->input, a->weight, out, seg_end, seg_end[2], a->k, LLMI_GEMV_OUT_BF16,
+                       static_cast<hipStream_t>(a->stream));
 }
 
 int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }

@@ -27,6 +27,8 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
 int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);
 int launch_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,
                         hipStream_t stream);
+int launch_gemv(const void* input, const void* weight, void* const out[3], const int32_t seg_end[3], int32_t n,
+                int32_t k, int32_t mode, hipStream_t stream);
 int launch_kv_restride(const void* src, void* dst, int32_t layer_num, int32_t max_seq_len,
                        int32_t kv_dim, int32_t head_dim, int32_t num_pos, hipStream_t stream);
 

@@ -140,3 +140,30 @@ def kv_restride(src_pos_major, dst_head_major, *, layer_num, max_seq_len, kv_dim
                                          max_seq_len, kv_dim, head_dim, num_pos, _stream_handle(stream)),
             "llmi_hip_kv_restride")
     return dst_head_major
+
+
+def gemv(input, weight, output, *, mode=B.GEMV_OUT_BF16, stream=None):
+    """output = weight @ input (bf16 [n][k] x bf16 [k], fp32 accumulate): bf16 or fp32 output, or the
+    bf16 residual in `output` updated in place (llmi_hip_gemv)."""
+    _check_dev("input", input, _BF16_DTYPES)
+    _check_dev("weight", weight, _BF16_DTYPES)
+    _check_dev("output", output, (torch.float32,) if mode == B.GEMV_OUT_F32 else _BF16_DTYPES)
+    a = B.GemvArgs()
+    a.input, a.weight, a.output = _ptr(input), _ptr(weight), _ptr(output)
+    a.n, a.k, a.mode = weight.shape[0], weight.shape[1], mode
+    a.stream = _stream_handle(stream)
+    B.check(B.lib().llmi_hip_gemv(ctypes.byref(a)), "llmi_hip_gemv")
+    return output
+
+
+def qkv_gemv(input, weight, query, key, value, *, stream=None):
+    """The packed QKV projection: rows [0, dim) of weight @ input go to query, the next kv_dim to key,
+    the last kv_dim to value (llmi_hip_qkv_gemv)."""
+    for name, t in (("input", input), ("weight", weight), ("query", query), ("key", key), ("value", value)):
+        _check_dev(name, t, _BF16_DTYPES)
+    a = B.QkvGemvArgs()
+    a.input, a.weight, a.query, a.key, a.value = _ptr(input), _ptr(weight), _ptr(query), _ptr(key), _ptr(value)
+    a.dim, a.kv_dim, a.k = query.numel(), key.numel(), weight.shape[1]
+    assert value.numel() == key.numel() and weight.shape[0] == a.dim + 2 * a.kv_dim
+    a.stream = _stream_handle(stream)
+    B.check(B.lib().llmi_hip_qkv_gemv(ctypes.byref(a)), "llmi_hip_qkv_gemv")

@@ -220,3 +220,33 @@ void llmi_oracle_qk_norm_rope(uint16_t* x, int32_t n_heads, int32_t head_dim,
         }
     }
 }
+
+/* code/source/op/kernel/cuda/matmul_kernel.cu:6-63 */
+void llmi_oracle_gemv_bf16(const uint16_t* x, const uint16_t* w, int32_t n, int32_t k,
+                           float* out) {
+    enum { kThreads = 256, kWarp = 32, kWarps = kThreads / kWarp };
+    const int32_t k8 = k / 8;                                   /* :46 */
+    for (int32_t r = 0; r < n; ++r) {
+        const uint16_t* wr = w + (size_t)r * (size_t)k;        /* :48 */
+        float part[kThreads];
+        for (int32_t t = 0; t < kThreads; ++t) {
+            float sum = 0.0f;                                   /* :50 */
+            for (int32_t i = t; i < k8; i += kThreads) {        /* :51 */
+                for (int32_t j = 0; j < 8; ++j) {               /* :57-60, pairs (x, y) in order */
+                    sum = fmaf(llmi_oracle_bf16_to_f32(x[i * 8 + j]), llmi_oracle_bf16_to_f32(wr[i * 8 + j]), sum);
+                }
+            }
+            part[t] = sum;
+        }
+        float warp_sum[kWarps];
+        for (int32_t wv = 0; wv < kWarps; ++wv) {               /* warp_reduce_sum<32>, :6-13 */
+            float* v = part + wv * kWarp;
+            for (int32_t delta = kWarp / 2; delta > 0; delta /= 2)
+                for (int32_t lane = 0; lane < delta; ++lane) v[lane] += v[lane + delta];
+            warp_sum[wv] = v[0];                                /* :21-23 */
+        }
+        for (int32_t delta = kWarps / 2; delta > 0; delta /= 2)  /* warp_reduce_sum<WARP_NUM>, :26-30 */
+            for (int32_t lane = 0; lane < delta; ++lane) warp_sum[lane] += warp_sum[lane + delta];
+        out[r] = warp_sum[0];
+    }
+}

@@ -97,6 +97,20 @@ void llmi_oracle_qk_norm_rope(uint16_t* x, int32_t n_heads, int32_t head_dim,
                               const uint16_t* weight, const float* sin_row,
                               const float* cos_row, float eps);
 
+/* bf16 GEMV of the layer's projections: out[r] = sum_k x[k] * w[r][k], fp32
+ * accumulate, in the order of the reference's 256-thread block
+ * (code/source/op/kernel/cuda/matmul_kernel.cu:38-63 with the block reduction
+ * :6-36): thread t adds the 8-element chunks t, t+256, ... left to right (the
+ * compiler's fused multiply-add), the 32 lanes of a warp fold by halving,
+ * then the 8 warp sums do. Result in fp32 (the lm_head variant, :65-98);
+ * llmi_oracle_f32_to_bf16 of it is the bf16 variant (:62), and
+ * f32_to_bf16(bf16_to_f32(residual[r]) + out[r]) the fused residual add
+ * (:143-172). The packed QKV GEMV (:211-246) is this routine on the weight
+ * [dim + 2*kv_dim][k] with the rows dealt to query, key and value.
+ * k must be a multiple of 8. */
+void llmi_oracle_gemv_bf16(const uint16_t* x, const uint16_t* w, int32_t n, int32_t k,
+                           float* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -61,6 +61,8 @@ def lib():
         L.llmi_oracle_qk_norm_rope.restype = None
         L.llmi_oracle_qk_norm_rope.argtypes = [_u16p, _i32, _i32, _u16p, _f32p, _f32p,
                                                ctypes.c_float]
+        L.llmi_oracle_gemv_bf16.restype = None
+        L.llmi_oracle_gemv_bf16.argtypes = [_u16p, _u16p, _i32, _i32, _f32p]
         _lib = L
     return _lib
 
@@ -166,3 +168,14 @@ def qk_norm_rope(x, weight, sin_row, cos_row, eps=1e-6):
     lib().llmi_oracle_qk_norm_rope(_u(y), y.shape[0], y.shape[1], _u(weight), _f(sin_row),
                                    _f(cos_row), eps)
     return y
+
+
+def gemv_bf16(x, w):
+    """x: uint16 [k], w: uint16 [n, k]; returns the fp32 sums [n] (before any output rounding)."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    w = np.ascontiguousarray(w, dtype=np.uint16)
+    n, k = w.shape
+    assert x.shape == (k,) and k % 8 == 0
+    out = np.empty(n, dtype=np.float32)
+    lib().llmi_oracle_gemv_bf16(_u(x), _u(w), n, k, _f(out))
+    return out

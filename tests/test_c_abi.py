@@ -196,3 +196,24 @@ def test_missing_library_fails_loudly(tmp_path):
             "try:\n    B.lib()\nexcept RuntimeError as e:\n    print('RAISED', e)\n" % (ROOT, str(tmp_path / "nope.so")))
     out = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, text=True, check=True).stdout
     assert "RAISED" in out and "no fallback" in out
+
+
+def test_gemv_argument_checks():
+    """Validation happens before any HIP call (k % 8, alignment: matmul_kernel.cu:123-128)."""
+    L = B.lib()
+    a = B.GemvArgs()
+    a.input, a.weight, a.output, a.n, a.k, a.mode = 0x1000, 0x2000, 0x3000, 16, 64, B.GEMV_OUT_BF16
+    for field, value, status in (("input", 0, "NULL_POINTER"), ("weight", 0, "NULL_POINTER"), ("output", 0, "NULL_POINTER"),
+                                 ("k", 60, "INVALID_ARG"), ("n", 0, "INVALID_ARG"), ("mode", 7, "INVALID_ARG"),
+                                 ("weight", 0x2008, "ALIGNMENT"), ("input", 0x1002, "ALIGNMENT")):
+        b = B.GemvArgs.from_buffer_copy(a)
+        setattr(b, field, value)
+        assert L.llmi_hip_gemv(ctypes.byref(b)) == B.STATUS[status], field
+    assert L.llmi_hip_gemv(None) == B.STATUS["NULL_POINTER"]
+    q = B.QkvGemvArgs()
+    q.input, q.weight, q.query, q.key, q.value, q.dim, q.kv_dim, q.k = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 256, 128, 64
+    for field, value, status in (("key", 0, "NULL_POINTER"), ("k", 4, "INVALID_ARG"), ("kv_dim", 0, "INVALID_ARG"),
+                                 ("value", 0x5004, "ALIGNMENT")):
+        b = B.QkvGemvArgs.from_buffer_copy(q)
+        setattr(b, field, value)
+        assert L.llmi_hip_qkv_gemv(ctypes.byref(b)) == B.STATUS[status], field

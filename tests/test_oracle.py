@@ -283,3 +283,45 @@ def test_qk_norm_rope_invariants(oracle):
     s3, c3 = float(sin[1, 3]), float(cos[1, 3])
     amp = np.sqrt(128.0)  # RMSNorm of a one-hot vector
     assert r[0, 3] == pytest.approx(amp * c3, rel=1e-2) and r[0, 67] == pytest.approx(amp * s3, rel=1e-2)
+
+
+# ---- bf16 GEMV (matmul_kernel.cu:6-63) --------------------------------------------------------------
+
+@pytest.mark.parametrize("n,k", [(7, 8), (5, 264), (3, 2048), (4, 2560), (2, 9728)])
+def test_gemv_against_float64(oracle, n, k):
+    """The restated 256-thread summation order against an exact float64 product: fp32 accumulation of k
+    exact products stays within k * 2^-24 of the sum of magnitudes (far inside: the tree keeps partial
+    sums short), and a transposed operand or a dropped chunk would miss by orders of magnitude."""
+    rng = np.random.RandomState(n * k)
+    x = synth.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))
+    w = synth.f32_to_bf16_bits(rng.standard_normal((n, k)).astype(np.float32))
+    xf, wf = synth.bf16_bits_to_f32(x).astype(np.float64), synth.bf16_bits_to_f32(w).astype(np.float64)
+    exact = wf @ xf
+    got = oracle.gemv_bf16(x, w)
+    assert np.all(np.abs(got - exact) <= 2e-6 * (np.abs(wf) @ np.abs(xf)))
+
+
+def test_gemv_exact_sums_and_one_hot(oracle):
+    k, n = 2048 + 264, 6
+    rng = np.random.RandomState(1)
+    w = synth.f32_to_bf16_bits(rng.standard_normal((n, k)).astype(np.float32))
+    for i in (0, 9, 2047, 2048, k - 1):                       # every thread slot and the ragged last sweep
+        x = np.zeros(k, dtype=np.float32)
+        x[i] = 1.0
+        assert np.array_equal(oracle.gemv_bf16(synth.f32_to_bf16_bits(x), w), synth.bf16_bits_to_f32(w[:, i]))
+    xi = rng.randint(-8, 9, size=k).astype(np.float32)
+    wi = rng.randint(-8, 9, size=(n, k)).astype(np.float32)  # integer sums are exact in any order
+    got = oracle.gemv_bf16(synth.f32_to_bf16_bits(xi), synth.f32_to_bf16_bits(wi))
+    assert np.array_equal(got, (wi.astype(np.float64) @ xi.astype(np.float64)).astype(np.float32))
+
+
+def test_gemv_matches_torch_bf16_matmul_rounding(oracle):
+    """Rounded to bf16 the result agrees with torch's fp32 matmul of the widened operands up to one step."""
+    import torch
+    rng = np.random.RandomState(5)
+    n, k = 64, 1024
+    x = synth.f32_to_bf16_bits(rng.standard_normal(k).astype(np.float32))
+    w = synth.f32_to_bf16_bits((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+    ref = (torch.from_numpy(synth.bf16_bits_to_f32(w)) @ torch.from_numpy(synth.bf16_bits_to_f32(x))).numpy()
+    got = oracle.gemv_bf16(x, w)
+    assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(synth.bf16_bits_to_f32(w)) @ np.abs(synth.bf16_bits_to_f32(x)))
