@@ -108,6 +108,82 @@ def cpu_baseline(ctx_list, budget_s=12.0, n_q=N_Q):
     }
 
 
+GEMV_SHAPES = {  # name -> (rows, k, what): the projections around the attention, Qwen3-4B (hidden 2560)
+    "qkv": (4096 + 2 * 1024, 2560, "packed QKV projection [dim + 2*kv_dim][hidden], rows dealt to q / k / v"),
+    "oproj": (2560, 4096, "output projection [hidden][dim] with the residual add folded in"),
+}
+
+
+def run_gemv(args):
+    """The bf16 GEMVs either side of the attention, each as a weight stream: 36 layers' worth of weights
+    (more than the 256 MB Infinity Cache) are walked in one HIP graph, like the layer loop does."""
+    import torch
+    from llminfer_amd import _binding as B
+    from llminfer_amd import ops
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    B.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n, k, what = GEMV_SHAPES[args.gemv]
+    layers = 36
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    w = (torch.randn((layers, n, k), generator=gen, device=dev) * 0.05).to(torch.bfloat16)
+    x = torch.randn(k, generator=gen, device=dev).to(torch.bfloat16)
+    q = torch.zeros(4096, dtype=torch.bfloat16, device=dev)
+    kk = torch.zeros(1024, dtype=torch.bfloat16, device=dev)
+    v = torch.zeros(1024, dtype=torch.bfloat16, device=dev)
+    res = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.Stream()
+
+    def enqueue():
+        for l in range(layers):
+            if args.gemv == "qkv":
+                ops.qkv_gemv(x, w[l], q, kk, v, stream=stream)
+            else:
+                ops.gemv(x, w[l], res, mode=B.GEMV_ADD_BF16, stream=stream)
+
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        enqueue()
+        stream.synchronize()
+        with torch.cuda.graph(g, stream=stream):
+            enqueue()
+
+    def timed(replays):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            e0.record(stream)
+            for _ in range(replays):
+                g.replay()
+            e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1)
+
+    timed(max(1, args.warmup // layers))
+    replays = max(1, args.steps // layers)
+    ms = timed(replays)
+    us = ms * 1e3 / (replays * layers)
+    # algorithmic bytes of one launch: the weight matrix once, the input, the output (read + written for the add)
+    nbytes = n * k * 2 + k * 2 + n * 2 * (2 if args.gemv == "oproj" else 1)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "bf16 GEMV around decode attention, us per launch + HBM GB/s", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": replays * layers, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s, %d x %d bf16, batch 1, 36 distinct weight matrices walked per HIP graph replay"
+                               % (what, n, k)},
+        "us_per_launch": round(us, 3),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "gemv_kernel",
+                     "avg_launch_us": round(us, 3), "avg_launch_bytes": nbytes},
+    }))
+    return 0
+
+
 def run_stack(args, ctx):
     """BASELINE config 4: the attention part of a 36-layer decode step at a fixed position, as one HIP graph."""
     import numpy as np
@@ -196,6 +272,8 @@ def main():
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
                     help="instead of the sweep: LAYERS layers of (QK-Norm + RoPE + append, attention) at --ctx (one "
                          "value) + 1 new token, captured into one HIP graph; reports us per token")
+    ap.add_argument("--gemv", choices=sorted(GEMV_SHAPES), default=None,
+                    help="time one of the GEMVs around the attention instead (Qwen3-4B shapes)")
     ap.add_argument("--stack-follow-pos", action="store_true",
                     help="with --stack: capture once for every position (kernels read it from device memory)")
     ap.add_argument("--stack-mode", type=int, default=2,
@@ -208,6 +286,8 @@ def main():
         return 2
     ctx_list = [int(c) for c in args.ctx.split(",")]
     n_q = args.heads
+    if args.gemv:
+        return run_gemv(args)
     if args.stack:
         return run_stack(args, ctx_list[0])
 

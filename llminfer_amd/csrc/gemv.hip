@@ -8,7 +8,10 @@
 // HBM-bound weight streams: every weight byte is read once, with non-temporal
 // 16-byte loads. A wavefront owns kRows consecutive rows and walks K in steps of
 // 512 elements (64 lanes x 8 bf16); the input chunk a lane needs is the same for all
-// of its rows and comes from L1/L2. Products are formed in fp32 by v_dot2_f32_bf16
+// of its rows and comes from L1/L2. Measured on the Qwen3-4B projections, many small
+// workgroups of one row per wavefront beat fewer, fatter ones (6144 x 2560: 7.1 vs
+// 7.7 us; 2560 x 4096: 5.6 vs 6.9 us): the matrices are a few microseconds of stream
+// and what counts is how fast the whole chip has loads in flight. Products are formed in fp32 by v_dot2_f32_bf16
 // (two bf16 pairs per instruction, fp32 accumulate), the 64 lanes fold with xor
 // shuffles, lane 0 rounds once and writes.
 
@@ -23,9 +26,18 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kRows = 4;    // rows per wavefront
-constexpr int kWaves = 4;   // wavefronts per workgroup
-constexpr int kUnroll = 2;  // K steps whose loads are issued together
+#ifndef LLMI_GEMV_ROWS
+#define LLMI_GEMV_ROWS 1
+#endif
+#ifndef LLMI_GEMV_UNROLL
+#define LLMI_GEMV_UNROLL 4
+#endif
+constexpr int kRows = LLMI_GEMV_ROWS;      // rows per wavefront
+#ifndef LLMI_GEMV_WAVES
+#define LLMI_GEMV_WAVES 2
+#endif
+constexpr int kWaves = LLMI_GEMV_WAVES;    // wavefronts per workgroup
+constexpr int kUnroll = LLMI_GEMV_UNROLL;  // K steps whose loads are issued together
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
 
