@@ -214,6 +214,10 @@ def run_stack(args, ctx):
         if rc != 0:
             raise RuntimeError(host.llmi_host_last_error().decode())
 
+    hidden = 2560 if n_q == 32 else 5120 if n_q == 64 else 1024
+    if args.stack_mode == 3:
+        host.llmi_host_stack_enable_projections.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+        ok(host.llmi_host_stack_enable_projections(st, hidden))
     ok(host.llmi_host_stack_build_sincos(st))
     rng = np.random.RandomState(4)
     rows = rng.standard_normal((msl * N_KV, HEAD_DIM)).astype(np.float32)
@@ -229,6 +233,18 @@ def run_stack(args, ctx):
         up(host.llmi_host_stack_ptr(st, 4, l), synth.f32_to_bf16_bits(rng.standard_normal(KV_DIM).astype(np.float32)))
         up(host.llmi_host_stack_ptr(st, 5, l),
            synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * HEAD_DIM)).astype(np.float32)))
+    if args.stack_mode == 3:
+        dim = n_q * HEAD_DIM
+        for l in range(layers):
+            up(host.llmi_host_stack_ptr(st, 12, l), synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32)))
+        # one random matrix of each kind, rolled per layer (the values do not matter to the stream, the
+        # addresses do: every layer reads its own 31 + 21 MB)
+        wqkv = synth.f32_to_bf16_bits((rng.standard_normal((dim + 2 * KV_DIM) * hidden) / np.sqrt(hidden)).astype(np.float32))
+        wo = synth.f32_to_bf16_bits((rng.standard_normal(hidden * dim) / np.sqrt(dim)).astype(np.float32))
+        for l in range(layers):
+            up(host.llmi_host_stack_ptr(st, 10, l), np.roll(wqkv, 8 * l))
+            up(host.llmi_host_stack_ptr(st, 11, l), np.roll(wo, 8 * l))
+        up(host.llmi_host_stack_ptr(st, 13, 0), synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32)))
     ok(host.llmi_host_stack_run(st, pos, args.stack_mode))
     if args.stack_follow_pos:
         host.llmi_host_stack_capture_following.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32]
@@ -242,6 +258,8 @@ def run_stack(args, ctx):
     ok(host.llmi_host_stack_replay(st, args.steps, ctypes.byref(ms)))
     us_token = ms.value * 1e3 / args.steps
     per_layer = algorithmic_bytes(pos + 1, n_q) + 23552  # + QK-Norm/RoPE/append traffic per layer
+    if args.stack_mode == 3:  # + both weight matrices, the hidden input and the residual (read + written)
+        per_layer += ((n_q * HEAD_DIM + 2 * KV_DIM) * hidden + hidden * n_q * HEAD_DIM) * 2 + 3 * hidden * 2
     gbs = layers * per_layer / (us_token * 1e-6) / 1e9
     host.llmi_host_stack_destroy(st)
     print(json.dumps({
@@ -251,7 +269,9 @@ def run_stack(args, ctx):
         "config": {"workload": "%d layers x (fused QK-Norm + RoPE + K/V append, GQA decode attention), %d Q / 8 KV "
                                "heads, ctx %d + 1 new token, one HIP graph per token, %s layout, %s"
                                % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major",
-                                  "one launch per layer" if args.stack_mode == 2 else "two launches per layer")
+                                  "one launch per layer" if args.stack_mode == 2 else
+                                  "three launches per layer: packed QKV GEMV (hidden %d), attention, output projection + "
+                                  "residual" % hidden if args.stack_mode == 3 else "two launches per layer")
                             + (", position read from device memory" if args.stack_follow_pos else "")},
         "us_per_layer": round(us_token / layers, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -277,7 +297,8 @@ def main():
     ap.add_argument("--stack-follow-pos", action="store_true",
                     help="with --stack: capture once for every position (kernels read it from device memory)")
     ap.add_argument("--stack-mode", type=int, default=2,
-                    help="with --stack: 2 = norm/rope/append fused into the attention launch (default), "
+                    help="with --stack: 3 = whole attention block (QKV GEMV, attention, o_proj + residual); "
+                         "2 = norm/rope/append fused into the attention launch (default), "
                          "1 = separate kernel before attention (the reference's sequence)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -34,6 +34,19 @@ DecodeStack::~DecodeStack() {
     if (graph_) (void)hipGraphDestroy(graph_);
 }
 
+void DecodeStack::enable_projections(int32_t hidden_dim) {
+    LLMI_CHECK(hidden_dim > 0 && hidden_dim % 8 == 0);
+    auto alloc = base::HIPDeviceAllocatorFactory::get_instance();
+    const int32_t L = config_.layer_num;
+    using base::DataType;
+    hidden_dim_ = hidden_dim;
+    wqkv_ = tensor::Tensor(DataType::DataTypeBf16, L, config_.dim() + 2 * config_.kv_dim(), hidden_dim, true, alloc);
+    wo_ = tensor::Tensor(DataType::DataTypeBf16, L, hidden_dim, config_.dim(), true, alloc);
+    hidden_ = tensor::Tensor(DataType::DataTypeBf16, L, hidden_dim, true, alloc);
+    residual_ = tensor::Tensor(DataType::DataTypeBf16, hidden_dim, true, alloc);
+    LLMI_CHECK(!wqkv_.is_empty() && !wo_.is_empty() && !hidden_.is_empty() && !residual_.is_empty());
+}
+
 void DecodeStack::build_sincos() {
     kernel::get_sin_cos_cache_kernel(base::DeviceType::DeviceHIP)(
         buffers_->get_buffer(ModelBufferType::SinCache), buffers_->get_buffer(ModelBufferType::CosCache),
@@ -44,6 +57,8 @@ void DecodeStack::build_sincos() {
 void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
     const bool with_qk_norm_rope = mode == kSeparateQkNormRope;
     LLMI_CHECK(!(follow_device_pos && with_qk_norm_rope));
+    const bool block = mode == kAttentionBlock;
+    LLMI_CHECK(!block || hidden_dim_ > 0);
     const AttentionConfig& c = config_;
     tensor::Tensor& kc = buffers_->get_buffer(ModelBufferType::KeyCache);
     tensor::Tensor& vc = buffers_->get_buffer(ModelBufferType::ValueCache);
@@ -75,6 +90,20 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
             if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_qk_norm_rope_append: " << llmi_hip_strerror(rc));
             q_for_attention = q.ptr<uint16_t>();
         }
+        if (block) {
+            llmi_qkv_gemv_args g{};
+            g.input = hidden_in(layer);
+            g.weight = qkv_weight(layer);
+            g.query = query_raw(layer);
+            g.key = key_raw(layer);
+            g.value = value_raw(layer);
+            g.dim = c.dim();
+            g.kv_dim = c.kv_dim();
+            g.k = hidden_dim_;
+            g.stream = stream();
+            const int rc = llmi_hip_qkv_gemv(&g);
+            if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_qkv_gemv: " << llmi_hip_strerror(rc));
+        }
         llmi_mha_args m{};
         m.query = q_for_attention;
         m.key_cache = kc.ptr<uint16_t>();
@@ -97,7 +126,7 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
         m.stream = stream();
         m.pos_device = follow_device_pos ? pos_dev_.ptr<int32_t>() : nullptr;
         int rc;
-        if (mode == kFusedAppend) {
+        if (mode == kFusedAppend || block) {
             llmi_mha_append_args f{};
             f.mha = m;
             f.mha.query = query_raw(layer);
@@ -112,6 +141,18 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
             rc = llmi_hip_mha_decode(&m);
         }
         if (rc != LLMI_OK) LLMI_FATAL("decode attention: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
+        if (block) {
+            llmi_gemv_args o{};
+            o.input = output(layer);
+            o.weight = out_weight(layer);
+            o.output = residual();
+            o.n = hidden_dim_;
+            o.k = c.dim();
+            o.mode = LLMI_GEMV_ADD_BF16;
+            o.stream = stream();
+            const int rc2 = llmi_hip_gemv(&o);
+            if (rc2 != LLMI_OK) LLMI_FATAL("llmi_hip_gemv: " << llmi_hip_strerror(rc2));
+        }
     }
 }
 

@@ -32,10 +32,23 @@ public:
     // Per-layer attention outputs [layer][dim], device bf16.
     uint16_t* output(int32_t layer) { return outputs_.ptr<uint16_t>(static_cast<int64_t>(layer) * config_.dim()); }
 
+    // Optional: the projections either side of the attention (packed QKV GEMV in front, output
+    // projection with residual add behind; code/source/model/qwen3_fused.cpp:517-553). Allocates
+    // per-layer weights [dim + 2*kv_dim][hidden] and [hidden][dim], per-layer inputs [hidden] and one
+    // residual stream [hidden]; needed by mode kAttentionBlock.
+    void enable_projections(int32_t hidden_dim);
+    int32_t hidden_dim() const { return hidden_dim_; }
+    uint16_t* qkv_weight(int32_t layer) { return wqkv_.ptr<uint16_t>(static_cast<int64_t>(layer) * (config_.dim() + 2 * config_.kv_dim()) * hidden_dim_); }
+    uint16_t* out_weight(int32_t layer) { return wo_.ptr<uint16_t>(static_cast<int64_t>(layer) * hidden_dim_ * config_.dim()); }
+    uint16_t* hidden_in(int32_t layer) { return hidden_.ptr<uint16_t>(static_cast<int64_t>(layer) * hidden_dim_); }
+    uint16_t* residual() { return residual_.ptr<uint16_t>(); }
+
     void build_sincos();
     // What one layer issues: attention alone on the raw query (0), the QK-Norm + RoPE + append kernel
     // followed by attention (1, the reference's sequence), or both fused into one launch (2).
-    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2 };
+    // kAttentionBlock (3): packed QKV GEMV -> fused append attention -> output projection + residual,
+    // three launches per layer.
+    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2, kAttentionBlock = 3 };
     // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
     // `follow_device_pos`: the kernels read the position from the stack's device word (set_position)
     // and `pos` is the largest position they may see; modes 0 and 2 only (the separate QK-Norm/RoPE
@@ -54,6 +67,8 @@ private:
     std::shared_ptr<kernel::HipConfig> hip_config_;
     std::unique_ptr<AttentionBuffers> buffers_;
     tensor::Tensor raw_q_, raw_k_, raw_v_, norm_w_, outputs_, pos_dev_;
+    tensor::Tensor wqkv_, wo_, hidden_, residual_;
+    int32_t hidden_dim_ = 0;
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
 };

@@ -64,10 +64,18 @@ void* llmi_host_stack_ptr(llmi_host_stack* s, int32_t which, int32_t layer) {
             case 7: p = d.buffers().get_buffer(ModelBufferType::SinCache).ptr<float>(); break;
             case 8: p = d.buffers().get_buffer(ModelBufferType::CosCache).ptr<float>(); break;
             case 9: p = d.buffers().get_buffer(ModelBufferType::Query).ptr<uint16_t>(); break;
+            case 10: p = d.qkv_weight(layer); break;
+            case 11: p = d.out_weight(layer); break;
+            case 12: p = d.hidden_in(layer); break;
+            case 13: p = d.residual(); break;
             default: LLMI_FATAL("unknown pointer selector " << which);
         }
     });
     return p;
+}
+
+int llmi_host_stack_enable_projections(llmi_host_stack* s, int32_t hidden_dim) {
+    return guarded([&] { s->impl->enable_projections(hidden_dim); });
 }
 
 int llmi_host_stack_build_sincos(llmi_host_stack* s) { return guarded([&] { s->impl->build_sincos(); }); }

@@ -19,10 +19,15 @@ llmi_host_stack* llmi_host_stack_create(int32_t layer_num, int32_t max_seq_len, 
                                         int32_t kv_head_num, int32_t kv_layout);
 void llmi_host_stack_destroy(llmi_host_stack* s);
 /* which: 0 key cache base, 1 value cache base, 2 raw query of `layer`, 3 raw key, 4 raw value,
- * 5 norm weight, 6 output of `layer`, 7 sin table, 8 cos table, 9 normalised query buffer. Device pointers. */
+ * 5 norm weight, 6 output of `layer`, 7 sin table, 8 cos table, 9 normalised query buffer; after
+ * llmi_host_stack_enable_projections: 10 packed QKV weight of `layer`, 11 output-projection weight, 12 hidden
+ * input of `layer`, 13 residual stream. Device pointers. */
 void* llmi_host_stack_ptr(llmi_host_stack* s, int32_t which, int32_t layer);
+/* Allocates the projections either side of the attention (mode 3: QKV GEMV, attention, o_proj + residual). */
+int llmi_host_stack_enable_projections(llmi_host_stack* s, int32_t hidden_dim);
 int llmi_host_stack_build_sincos(llmi_host_stack* s);
-/* with_qk_norm_rope: 0 attention only, 1 separate QK-Norm/RoPE/append kernel + attention, 2 both fused */
+/* with_qk_norm_rope: 0 attention only, 1 separate QK-Norm/RoPE/append kernel + attention, 2 both fused,
+ * 3 the whole attention block (packed QKV GEMV, fused append attention, output projection + residual) */
 int llmi_host_stack_run(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);      /* eager + synchronise */
 int llmi_host_stack_capture(llmi_host_stack* s, int32_t pos, int32_t with_qk_norm_rope);
 int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms);

@@ -368,6 +368,68 @@ def test_decode_stack_graph_follows_the_device_position(oracle, dev):
         H.L.llmi_host_stack_destroy(stack)
 
 
+def test_attention_block_stack_matches_the_oracle_chain(oracle, dev):
+    """Mode 3 of the stack, two layers: packed QKV GEMV -> QK-Norm + RoPE + append + attention -> output
+    projection added to the residual stream. The oracle replays the chain with a bf16 rounding wherever
+    the kernels store bf16 (GEMV outputs, attention output, residual)."""
+    H = HostLib()
+    H.L.llmi_host_stack_enable_projections.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+    layers, ctx, n_q, n_kv, d, hidden, layout = 2, 280, 16, 8, 128, 1024, B.KV_LAYOUT_HEAD_MAJOR
+    dim, kv_dim, msl, pos = n_q * d, n_kv * d, ctx + 1, ctx
+    stack = H.L.llmi_host_stack_create(layers, msl, n_q, n_kv, layout)
+    assert stack, H.L.llmi_host_last_error().decode()
+    try:
+        H.ok(H.L.llmi_host_stack_enable_projections(stack, hidden))
+        H.ok(H.L.llmi_host_stack_build_sincos(stack))
+        rng = np.random.RandomState(21)
+        sin_o, cos_o = oracle.sincos_table(d, msl)
+        k_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        v_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
+        res0 = synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32))
+        res_ref = synth.bf16_bits_to_f32(res0).copy()
+        attn_refs = []
+        for l in range(layers):
+            c = synth.make_case(800 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+            k_all[l], v_all[l] = c["k"][0], c["v"][0]
+            x = synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32))
+            wqkv = synth.f32_to_bf16_bits((rng.standard_normal((dim + 2 * kv_dim, hidden)) / np.sqrt(hidden)).astype(np.float32))
+            wo = synth.f32_to_bf16_bits((rng.standard_normal((hidden, dim)) / np.sqrt(dim)).astype(np.float32))
+            w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+            for which, arr in ((12, x), (10, wqkv), (11, wo), (5, w)):
+                _upload(H.L.llmi_host_stack_ptr(stack, which, l), arr)
+            qkv = synth.f32_to_bf16_bits(oracle.gemv_bf16(x, wqkv))
+            qr, kr, vr = qkv[:dim].reshape(n_q, d), qkv[dim:dim + kv_dim].reshape(n_kv, d), qkv[dim + kv_dim:]
+            k_all[l, pos] = oracle.qk_norm_rope(kr, w[d:], sin_o[pos], cos_o[pos]).reshape(-1)
+            v_all[l, pos] = vr
+            qn = oracle.qk_norm_rope(qr, w[:d], sin_o[pos], cos_o[pos]).reshape(-1)
+            attn = oracle.mha_cpu(qn, k_all[l:l + 1], v_all[l:l + 1], 0, pos, kv_dim, n_q // n_kv, n_q, d, msl)
+            attn_refs.append(attn)
+            proj = oracle.gemv_bf16(synth.f32_to_bf16_bits(attn), wo)
+            res_ref = synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(res_ref + proj))
+        k_up = k_all.copy()
+        v_up = v_all.copy()
+        k_up[:, pos], v_up[:, pos] = 0x7FC0, 0x7FC0  # the new rows are the kernels' to write
+        _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), synth.to_head_major(k_up, n_kv))
+        _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), synth.to_head_major(v_up, n_kv))
+        _upload(H.L.llmi_host_stack_ptr(stack, 13, 0), res0)
+        H.ok(H.L.llmi_host_stack_run(stack, pos, 3))
+        for l in range(layers):
+            got = _download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16)
+            assert_parity(synth.bf16_bits_to_f32(got), attn_refs[l], "block layer %d attention" % l)
+        res = synth.bf16_bits_to_f32(_download(H.L.llmi_host_stack_ptr(stack, 13, 0), (hidden,), np.uint16))
+        # residual of magnitude ~1: one bf16 step is 2^-8 relative; the projections add O(1) values
+        assert np.all(np.abs(res - res_ref) <= np.abs(res_ref) / 64 + 2e-2), np.abs(res - res_ref).max()
+        # graph replay of the block gives the same residual increment again
+        _upload(H.L.llmi_host_stack_ptr(stack, 13, 0), res0)
+        H.ok(H.L.llmi_host_stack_capture(stack, pos, 3))
+        ms = ctypes.c_float()
+        H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
+        res2 = synth.bf16_bits_to_f32(_download(H.L.llmi_host_stack_ptr(stack, 13, 0), (hidden,), np.uint16))
+        assert np.array_equal(res, res2)
+    finally:
+        H.L.llmi_host_stack_destroy(stack)
+
+
 def test_mha_op_forward_through_registry_hook(oracle, dev):
     """op::MultiHeadAttention::forward (C++ op layer -> registry -> HIP arm) on borrowed device tensors."""
     H = HostLib()
