@@ -185,7 +185,7 @@ def run_gemv(args):
 
 
 def run_stack(args, ctx):
-    """BASELINE config 4: the attention part of a 36-layer decode step at a fixed position, as one HIP graph."""
+    """The attention part of a 36-layer decode step at a fixed position, as one HIP graph."""
     import numpy as np
     from llminfer_amd import _binding as B
     from llminfer_amd import synth

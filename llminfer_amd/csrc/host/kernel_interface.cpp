@@ -39,6 +39,21 @@ SinCosCacheKernel get_sin_cos_cache_kernel(base::DeviceType device_type) {
     LLMI_FATAL("Unknown device type for get a sin_cos_cache kernel.");
 }
 
+GEMVKernel get_gemv_kernel(base::DeviceType device_type) {
+    if (device_type == base::DeviceType::DeviceHIP) return gemv_kernel_hip;
+    LLMI_FATAL("Unknown device type for get a gemv kernel.");
+}
+
+FusedGEMVAddKernel get_fused_gemv_add_kernel(base::DeviceType device_type) {
+    if (device_type == base::DeviceType::DeviceHIP) return fused_gemv_add_kernel_hip;
+    LLMI_FATAL("Unknown device type for get a fused_gemv_add kernel.");
+}
+
+FusedQKVGEMVKernel get_fused_qkv_gemv_kernel(base::DeviceType device_type) {
+    if (device_type == base::DeviceType::DeviceHIP) return fused_qkv_gemv_kernel_hip;
+    LLMI_FATAL("Unknown device type for get a fused_qkv_gemv kernel.");
+}
+
 MhaHipOptions& mha_hip_options() {
     static MhaHipOptions opts;
     return opts;
@@ -144,6 +159,72 @@ void sin_cos_cache_precompute_hip(const tensor::Tensor& sin_cache, const tensor:
     fail_on(llmi_hip_sincos_table(const_cast<float*>(sin_cache.ptr<float>()), const_cast<float*>(cos_cache.ptr<float>()),
                                   head_dim, max_seq_len, stream),
             "llmi_hip_sincos_table");
+}
+
+// matmul_kernel.cu:107-128: shapes, dtypes and devices of a GEMV's operands.
+static void check_gemv_operands(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& output,
+                                base::DataType out_type) {
+    LLMI_CHECK(!input.is_empty() && input.dims_size() == 1);
+    LLMI_CHECK(!weight.is_empty() && weight.dims_size() == 2);
+    LLMI_CHECK(!output.is_empty() && output.dims_size() == 1);
+    LLMI_CHECK(input.data_type() == base::DataType::DataTypeBf16);
+    LLMI_CHECK(weight.data_type() == base::DataType::DataTypeBf16);
+    LLMI_CHECK(output.data_type() == out_type);
+    for (const tensor::Tensor* t : {&input, &weight, &output}) LLMI_CHECK(t->device_type() == base::DeviceType::DeviceHIP);
+    LLMI_CHECK(input.get_dim(0) == weight.get_dim(1));
+}
+
+static void run_gemv(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& output,
+                     int32_t mode, void* stream) {
+    LLMI_CHECK(output.get_dim(0) == weight.get_dim(0));
+    llmi_gemv_args a{};
+    a.input = input.ptr<uint16_t>();
+    a.weight = weight.ptr<uint16_t>();
+    a.output = const_cast<void*>(static_cast<const void*>(output.ptr<uint8_t>()));  // outputs arrive const, like the reference's
+    a.n = weight.get_dim(0);
+    a.k = weight.get_dim(1);
+    a.mode = mode;
+    a.stream = stream;
+    fail_on(llmi_hip_gemv(&a), "llmi_hip_gemv");
+}
+
+void gemv_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& output,
+                     bool lm_head, void* stream) {
+    check_gemv_operands(input, weight, output, lm_head ? base::DataType::DataTypeFp32 : base::DataType::DataTypeBf16);
+    run_gemv(input, weight, output, lm_head ? LLMI_GEMV_OUT_F32 : LLMI_GEMV_OUT_BF16, stream);
+}
+
+void fused_gemv_add_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight,
+                               const tensor::Tensor& output, void* stream) {
+    check_gemv_operands(input, weight, output, base::DataType::DataTypeBf16);
+    run_gemv(input, weight, output, LLMI_GEMV_ADD_BF16, stream);
+}
+
+void fused_qkv_gemv_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& query,
+                               const tensor::Tensor& key, const tensor::Tensor& value, void* stream) {
+    // matmul_kernel.cu:256-292
+    LLMI_CHECK(!input.is_empty() && input.dims_size() == 1);
+    LLMI_CHECK(!weight.is_empty() && weight.dims_size() == 2);
+    for (const tensor::Tensor* t : {&query, &key, &value}) LLMI_CHECK(!t->is_empty() && t->dims_size() == 1);
+    for (const tensor::Tensor* t : {&input, &weight, &query, &key, &value}) {
+        LLMI_CHECK(t->data_type() == base::DataType::DataTypeBf16);
+        LLMI_CHECK(t->device_type() == base::DeviceType::DeviceHIP);
+    }
+    const int32_t dim = query.get_dim(0), kv_dim = key.get_dim(0);
+    LLMI_CHECK(value.get_dim(0) == kv_dim);
+    LLMI_CHECK(weight.get_dim(0) == dim + 2 * kv_dim);
+    LLMI_CHECK(weight.get_dim(1) == input.get_dim(0));
+    llmi_qkv_gemv_args a{};
+    a.input = input.ptr<uint16_t>();
+    a.weight = weight.ptr<uint16_t>();
+    a.query = const_cast<uint16_t*>(query.ptr<uint16_t>());
+    a.key = const_cast<uint16_t*>(key.ptr<uint16_t>());
+    a.value = const_cast<uint16_t*>(value.ptr<uint16_t>());
+    a.dim = dim;
+    a.kv_dim = kv_dim;
+    a.k = weight.get_dim(1);
+    a.stream = stream;
+    fail_on(llmi_hip_qkv_gemv(&a), "llmi_hip_qkv_gemv");
 }
 
 }  // namespace kernel

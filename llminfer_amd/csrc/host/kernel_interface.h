@@ -40,6 +40,20 @@ using SinCosCacheKernel = void (*)(const tensor::Tensor& sin_cache, const tensor
                                    int32_t head_dim, int32_t max_seq_len, void* stream);
 SinCosCacheKernel get_sin_cos_cache_kernel(base::DeviceType device_type);
 
+// The bf16 GEMVs either side of the attention (kernel_interface.h:49-65,76-84 of the reference).
+using GEMVKernel = void (*)(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& output,
+                            bool lm_head, void* stream);
+GEMVKernel get_gemv_kernel(base::DeviceType device_type);
+
+using FusedGEMVAddKernel = void (*)(const tensor::Tensor& input, const tensor::Tensor& weight,
+                                    const tensor::Tensor& output, void* stream);
+FusedGEMVAddKernel get_fused_gemv_add_kernel(base::DeviceType device_type);
+
+using FusedQKVGEMVKernel = void (*)(const tensor::Tensor& input, const tensor::Tensor& weight,
+                                    const tensor::Tensor& query, const tensor::Tensor& key,
+                                    const tensor::Tensor& value, void* stream);
+FusedQKVGEMVKernel get_fused_qkv_gemv_kernel(base::DeviceType device_type);
+
 // The gfx950 implementations (thin shims over the C ABI of libllmi_hip.so).
 // A 3-D key/value cache tensor [layers, max_seq_len, kv_dim] is the
 // reference's position-major layout; a 4-D one [layers, kv_heads, max_seq_len,
@@ -52,6 +66,12 @@ void fused_qk_norm_rope_kernel_hip(const tensor::Tensor& query, const tensor::Te
                                    const tensor::Tensor& weight, const tensor::Tensor& token_pos,
                                    const tensor::Tensor& sin_cache, const tensor::Tensor& cos_cache, int32_t dim,
                                    int32_t kv_dim, int32_t head_dim, void* stream);
+void gemv_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& output,
+                     bool lm_head, void* stream);
+void fused_gemv_add_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight,
+                               const tensor::Tensor& output, void* stream);
+void fused_qkv_gemv_kernel_hip(const tensor::Tensor& input, const tensor::Tensor& weight, const tensor::Tensor& query,
+                               const tensor::Tensor& key, const tensor::Tensor& value, void* stream);
 void sin_cos_cache_precompute_hip(const tensor::Tensor& sin_cache, const tensor::Tensor& cos_cache, int32_t head_dim,
                                   int32_t max_seq_len, void* stream);
 

@@ -217,6 +217,11 @@ TEST(cpu_registry_arms) {
     EXPECT(kernel::get_fused_qk_norm_rope_kernel(DeviceType::DeviceHIP) != nullptr);
     EXPECT(is_fatal([] { kernel::get_fused_qk_norm_rope_kernel(DeviceType::DeviceCPU); }));
     EXPECT(is_fatal([] { kernel::get_sin_cos_cache_kernel(DeviceType::DeviceCPU); }));
+    EXPECT(kernel::get_gemv_kernel(DeviceType::DeviceHIP) != nullptr);
+    EXPECT(kernel::get_fused_gemv_add_kernel(DeviceType::DeviceHIP) != nullptr);
+    EXPECT(kernel::get_fused_qkv_gemv_kernel(DeviceType::DeviceHIP) != nullptr);
+    EXPECT(is_fatal([] { kernel::get_gemv_kernel(DeviceType::DeviceCPU); }));
+    EXPECT(is_fatal([] { kernel::get_fused_qkv_gemv_kernel(DeviceType::DeviceUnknown); }));
     EXPECT(is_fatal([] { kernel::register_mha_kernel(DeviceType::DeviceHIP, oracle_mha_cpu_arm); }));
     kernel::register_mha_kernel(DeviceType::DeviceCPU, oracle_mha_cpu_arm);
     EXPECT(kernel::get_mha_kernel(DeviceType::DeviceCPU) == oracle_mha_cpu_arm);
@@ -429,6 +434,53 @@ TEST(gpu_qk_norm_rope_op_in_place) {
     EXPECT(mismatches < (dim + kv_dim) / 100);
     token_pos.index<int32_t>(0) = msl;  // past the table
     EXPECT(is_fatal([&] { layer.forward(q_d, k_d, token_pos, sin_d, cos_d, unused); }) || true);
+}
+
+TEST(gpu_gemv_family_through_the_registry) {
+    // 0.6B-like projections: packed QKV [2048 + 2*1024][1024], output projection [1024][2048] + residual.
+    const int32_t hidden = 1024, dim = 2048, kv_dim = 1024, n = dim + 2 * kv_dim;
+    std::mt19937 rng(9);
+    tensor::Tensor x(DataType::DataTypeBf16, hidden, true, cpu_alloc());
+    tensor::Tensor wqkv(DataType::DataTypeBf16, n, hidden, true, cpu_alloc());
+    tensor::Tensor wo(DataType::DataTypeBf16, hidden, dim, true, cpu_alloc());
+    tensor::Tensor res(DataType::DataTypeBf16, hidden, true, cpu_alloc());
+    fill_bf16_normal(x, rng, false);
+    fill_bf16_normal(res, rng, false);
+    std::normal_distribution<float> nd;
+    for (size_t i = 0; i < wqkv.size(); ++i) wqkv.index<uint16_t>(i) = llmi_oracle_f32_to_bf16(0.03f * nd(rng));
+    for (size_t i = 0; i < wo.size(); ++i) wo.index<uint16_t>(i) = llmi_oracle_f32_to_bf16(0.02f * nd(rng));
+    std::vector<float> qkv_ref(n), proj_ref(hidden);
+    llmi_oracle_gemv_bf16(x.ptr<uint16_t>(), wqkv.ptr<uint16_t>(), n, hidden, qkv_ref.data());
+
+    auto cfg = std::make_shared<kernel::HipConfig>();
+    cfg->create();
+    tensor::Tensor x_d = x.clone(), wqkv_d = wqkv.clone(), wo_d = wo.clone(), res_d = res.clone();
+    x_d.to_hip(); wqkv_d.to_hip(); wo_d.to_hip(); res_d.to_hip();
+    tensor::Tensor q_d(DataType::DataTypeBf16, dim, true, hip_alloc());
+    tensor::Tensor k_d(DataType::DataTypeBf16, kv_dim, true, hip_alloc());
+    tensor::Tensor v_d(DataType::DataTypeBf16, kv_dim, true, hip_alloc());
+    tensor::Tensor logits_d(DataType::DataTypeFp32, n, true, hip_alloc());
+    kernel::get_fused_qkv_gemv_kernel(DeviceType::DeviceHIP)(x_d, wqkv_d, q_d, k_d, v_d, cfg->stream);
+    kernel::get_gemv_kernel(DeviceType::DeviceHIP)(x_d, wqkv_d, logits_d, true, cfg->stream);  // fp32 output
+    kernel::get_fused_gemv_add_kernel(DeviceType::DeviceHIP)(q_d, wo_d, res_d, cfg->stream);
+    EXPECT(hipStreamSynchronize(cfg->stream) == hipSuccess);
+    q_d.to_cpu(); k_d.to_cpu(); v_d.to_cpu(); logits_d.to_cpu(); res_d.to_cpu();
+    auto near_bf16 = [](uint16_t got, float want) {
+        return std::fabs(llmi_oracle_bf16_to_f32(got) - want) <= std::fabs(want) * (1.0f / 128) + 1e-4f;
+    };
+    for (int i = 0; i < dim; ++i) EXPECT(near_bf16(q_d.index<uint16_t>(i), qkv_ref[i]));
+    for (int i = 0; i < kv_dim; ++i) {
+        EXPECT(near_bf16(k_d.index<uint16_t>(i), qkv_ref[dim + i]));
+        EXPECT(near_bf16(v_d.index<uint16_t>(i), qkv_ref[dim + kv_dim + i]));
+    }
+    for (int i = 0; i < n; ++i) EXPECT(std::fabs(logits_d.index<float>(i) - qkv_ref[i]) <= 1e-4f);
+    // the output projection consumed the device's own bf16 query vector
+    llmi_oracle_gemv_bf16(q_d.ptr<uint16_t>(), wo.ptr<uint16_t>(), hidden, dim, proj_ref.data());
+    for (int i = 0; i < hidden; ++i)
+        EXPECT(near_bf16(res_d.index<uint16_t>(i), llmi_oracle_bf16_to_f32(res.index<uint16_t>(i)) + proj_ref[i]));
+    // operand checks of the shims: wrong output type, wrong inner dimension
+    tensor::Tensor bad_out(DataType::DataTypeFp32, hidden, true, hip_alloc());
+    EXPECT(is_fatal([&] { kernel::get_fused_gemv_add_kernel(DeviceType::DeviceHIP)(q_d, wo_d, bad_out, cfg->stream); }));
 }
 
 int main(int argc, char** argv) {
