@@ -23,10 +23,10 @@ thread_local std::string g_last_error;
 // Context lengths up to this run as one workgroup per KV head; longer ones are
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
-// memory round trips for its combine, about 3 us, while one workgroup streams a
-// whole KV head at 16 tiles in about 7 us: measured crossover between 192 and
-// 256 positions at 32 query / 8 KV heads.)
-constexpr int kSinglePassMaxLen = 240;
+// memory round trips for its combine, while one workgroup of 8 waves streams a
+// whole KV head of 19 tiles in about 7 us: measured at 32 query / 8 KV heads.)
+constexpr int kSinglePassMaxLen8 = 304;  // single pass wins up to here with 8 waves (7.0 vs 7.3 us at 288)
+constexpr int kSinglePassMaxLen4 = 272;  // ... and up to here when only 4 waves are available (7.2 vs 7.3 us)
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).
@@ -105,11 +105,13 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
     // fused combine: per head and split, 128 partial outputs and two 8-byte arrival records
     const size_t per_split_fused = (size_t)a->head_num * (a->head_dim * sizeof(float) + 2 * sizeof(unsigned long long));
 
+    const int single_waves_max = (max_waves < wave_cap ? max_waves : wave_cap);  // 8 where the kernel variant allows
+    const int single_pass_max = single_waves_max >= 8 ? kSinglePassMaxLen8 : kSinglePassMaxLen4;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
         else if (a->num_splits > 1) path = LLMI_PATH_SPLIT;
-        else path = seq_len <= kSinglePassMaxLen ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT_FUSED;
+        else path = seq_len <= single_pass_max ? LLMI_PATH_SINGLE_PASS : LLMI_PATH_SPLIT_FUSED;
         if (path == LLMI_PATH_SPLIT) path = LLMI_PATH_SPLIT_FUSED;
     }
     // The separate combine kernel takes its split count from the launch, not from the device.
@@ -160,8 +162,7 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             waves = a->waves_per_group;
         } else {
             waves = pow2_ceil(tiles);
-            if (waves > kAutoMaxWaves) waves = kAutoMaxWaves;
-            if (waves > max_waves) waves = max_waves;
+            if (waves > single_waves_max) waves = single_waves_max;
         }
     }
 

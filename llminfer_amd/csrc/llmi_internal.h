@@ -12,7 +12,6 @@ constexpr int kMaxSplits = 256;     // upper bound on the KV split count
 constexpr int kMaxGroup = 16;       // query heads per KV head the kernels accept
 constexpr int kMaxGroupWaves = 64;  // group_pad * waves_per_group that fits the LDS merge
 constexpr int kMaxWaves = 8;        // wavefronts per workgroup the kernels are instantiated for
-constexpr int kAutoMaxWaves = 4;    // what the dispatcher picks by itself (two 8 KiB LDS stages per wave in 64 KiB)
 
 // Records a failed HIP call for llmi_hip_last_error() and maps it to LLMI_ERR_LAUNCH.
 int record_hip_error(hipError_t err, const char* what);
