@@ -47,6 +47,31 @@ void DecodeStack::enable_projections(int32_t hidden_dim) {
     LLMI_CHECK(!wqkv_.is_empty() && !wo_.is_empty() && !hidden_.is_empty() && !residual_.is_empty());
 }
 
+base::Status DecodeStack::load_weights(const WeightFile& file) {
+    const ModelConfig& f = file.config();
+    const AttentionConfig& c = config_;
+    if (f.head_num != c.head_num || f.kv_head_num != c.kv_head_num || file.head_dim() != c.head_dim)
+        return base::error::invalid_argument("The weight file's head layout differs from the stack's.");
+    if (f.layer_num < c.layer_num) return base::error::invalid_argument("The weight file has fewer layers than the stack.");
+    if (hidden_dim_ == 0) enable_projections(f.hidden_dim);
+    if (hidden_dim_ != f.hidden_dim) return base::error::invalid_argument("The weight file's hidden_dim differs from the stack's.");
+    const size_t qkv_bytes = static_cast<size_t>(c.dim() + 2 * c.kv_dim()) * hidden_dim_ * sizeof(uint16_t);
+    const size_t o_bytes = static_cast<size_t>(hidden_dim_) * c.dim() * sizeof(uint16_t);
+    const size_t norm_bytes = 2 * static_cast<size_t>(c.head_dim) * sizeof(uint16_t);
+    for (int32_t l = 0; l < c.layer_num; ++l) {
+        const std::pair<void*, std::pair<const void*, size_t>> copies[] = {
+            {qkv_weight(l), {file.qkv_proj(l), qkv_bytes}},
+            {norm_weight(l), {file.qk_norm(l), norm_bytes}},
+            {out_weight(l), {file.o_proj(l), o_bytes}},
+        };
+        for (const auto& cp : copies) {
+            const int rc = llmi_hip_memcpy(cp.first, cp.second.first, cp.second.second, 1, nullptr, 1);  // host to device
+            if (rc != LLMI_OK) return base::error::internal_error(std::string("weight upload: ") + llmi_hip_strerror(rc));
+        }
+    }
+    return base::error::success();
+}
+
 void DecodeStack::build_sincos() {
     kernel::get_sin_cos_cache_kernel(base::DeviceType::DeviceHIP)(
         buffers_->get_buffer(ModelBufferType::SinCache), buffers_->get_buffer(ModelBufferType::CosCache),

@@ -12,6 +12,7 @@
 
 #include "attention_buffers.h"
 #include "hip_config.h"
+#include "weight_file.h"
 
 namespace model {
 
@@ -42,6 +43,11 @@ public:
     uint16_t* out_weight(int32_t layer) { return wo_.ptr<uint16_t>(static_cast<int64_t>(layer) * hidden_dim_ * config_.dim()); }
     uint16_t* hidden_in(int32_t layer) { return hidden_.ptr<uint16_t>(static_cast<int64_t>(layer) * hidden_dim_); }
     uint16_t* residual() { return residual_.ptr<uint16_t>(); }
+
+    // Uploads the attention block's weights of every layer of this stack from a mapped weight file
+    // (packed QKV projection, q_norm/k_norm, output projection); enables the projections if needed.
+    // The file must describe the stack's head layout; it may hold more layers than the stack.
+    base::Status load_weights(const WeightFile& file);
 
     void build_sincos();
     // What one layer issues: attention alone on the raw query (0), the QK-Norm + RoPE + append kernel

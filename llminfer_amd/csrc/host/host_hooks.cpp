@@ -1,5 +1,6 @@
 #include "host_hooks.h"
 
+#include <cstring>
 #include <string>
 
 #include "decode_stack.h"
@@ -104,6 +105,44 @@ int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms)
         const float ms = s->impl->replay(times);
         if (elapsed_ms) *elapsed_ms = ms;
     });
+}
+
+int llmi_host_stack_load_weights(llmi_host_stack* s, const char* path) {
+    int code = -1;
+    const int rc = guarded([&] {
+        std::unique_ptr<model::WeightFile> file;
+        base::Status st = model::WeightFile::open(path ? path : "", &file);
+        if (st) st = s->impl->load_weights(*file);
+        code = int(st);
+        if (!st) g_err = st.get_err_msg();
+    });
+    return rc != 0 ? rc : code;
+}
+
+int llmi_host_weight_file_info(const char* path, int32_t header_ints, int64_t info[12], void* payload_out,
+                               int64_t payload_bytes) {
+    int code = -1;
+    std::string msg;
+    const int rc = guarded([&] {
+        std::unique_ptr<model::WeightFile> file;
+        const base::Status st = model::WeightFile::open(path ? path : "", &file, header_ints);
+        code = int(st);
+        msg = st.get_err_msg();
+        if (!st) return;
+        const model::ModelConfig& c = file->config();
+        const int32_t raw[8] = {c.dim, c.hidden_dim, c.layer_num, c.head_num, c.kv_head_num, c.vocab_size, c.max_seq_len, c.immediate_dim};
+        for (int i = 0; i < 8; ++i) info[i] = raw[i];
+        info[8] = file->head_dim();
+        info[9] = file->kv_dim();
+        info[10] = file->vocab_size();
+        info[11] = static_cast<int64_t>(file->payload_elements());
+        if (payload_out && payload_bytes > 0) {
+            const size_t have = file->payload_elements() * sizeof(uint16_t);
+            std::memcpy(payload_out, file->payload_bytes(), static_cast<size_t>(payload_bytes) < have ? static_cast<size_t>(payload_bytes) : have);
+        }
+    });
+    if (rc == 0 && code != 0) g_err = msg;
+    return rc != 0 ? rc : code;
 }
 
 void llmi_host_set_mha_options(int32_t force_path, int32_t num_splits, int32_t waves_per_group) {

@@ -35,6 +35,13 @@ int llmi_host_stack_replay(llmi_host_stack* s, int32_t times, float* elapsed_ms)
  * (llmi_mha_args.pos_device) that llmi_host_stack_set_pos writes between replays. mode 0 or 2. */
 int llmi_host_stack_capture_following(llmi_host_stack* s, int32_t max_pos, int32_t mode);
 int llmi_host_stack_set_pos(llmi_host_stack* s, int32_t pos);
+/* Loads the attention block's weights of every layer from an engine weight file (model::WeightFile). */
+int llmi_host_stack_load_weights(llmi_host_stack* s, const char* path);
+/* Opens a weight file (header_ints 8, or 7 for the older header) and reports: info[0..7] the header as stored,
+ * info[8] head_dim, info[9] kv_dim, info[10] |vocab_size|, info[11] payload elements (bf16). Copies up to
+ * payload_bytes of the payload to payload_out. Returns the base::Status code (0 success, 2 path, 3 parse). */
+int llmi_host_weight_file_info(const char* path, int32_t header_ints, int64_t info[12], void* payload_out,
+                               int64_t payload_bytes);
 /* Process-wide tuning overrides of the HIP attention arm (0 = automatic). */
 void llmi_host_set_mha_options(int32_t force_path, int32_t num_splits, int32_t waves_per_group);
 
