@@ -6,31 +6,39 @@
 //     KV head and writes the bf16 result itself;
 //   * KV split     (num_splits  > 1): workgroup (split, kv_head) owns a
 //     contiguous range of positions and leaves (o[128], m, l) per query head
-//     in the fp32 workspace; mha_combine_kernel merges them (log-sum-exp).
+//     in the fp32 workspace; either mha_combine_kernel merges them
+//     (log-sum-exp, a second launch) or the workgroup of the last split does,
+//     inside the same launch (fused combine).
+// Two more template switches: APPEND folds the per-token QK-Norm + RoPE and the
+// K/V cache append of the reference's layer loop into the launch, DYN reads the
+// position from device memory so that one captured launch serves every token.
 //
 // Differences from the reference design, chosen for CDNA4:
 //   * a workgroup serves ALL query heads of its KV head, so K and V are read
 //     from HBM exactly once (the reference re-reads them once per query head,
 //     mha_kernel.cu:67,104);
+//   * K/V tiles stream through per-wave LDS rings filled by LDS-DMA loads;
 //   * q.K^T runs on the matrix cores: one v_mfma_f32_16x16x32_bf16 chain per
-//     tile of 16 positions, K rows as the A operand straight from 16-byte
-//     global loads (lane = row, no LDS transpose needed because the
-//     contraction over head_dim is order-free), the query group as B;
-//   * p.V stays on the vector ALU in fp32 (p is never rounded to bf16): each
-//     16-lane DPP row owns 4 positions of the tile and 128 output columns,
-//     and picks its softmax weights out of the MFMA result layout with
-//     row_newbcast -- no LDS traffic in the inner loop;
+//     tile of 16 positions, K rows as the A operand (lane = row, no transpose
+//     needed because the contraction over head_dim is order-free), the query
+//     group as B;
+//   * P^T.V runs on the matrix cores too (v_mfma_f32_16x16x16_bf16): the score
+//     MFMA leaves a lane's four probabilities exactly where the A fragment of
+//     that product wants them, the V fragment is packed from the lane's four
+//     16-byte V rows with v_perm_b32; a probability enters as hi + lo bf16, so
+//     the product is as accurate as an fp32 one;
 //   * running max / sum are kept in the exp2 domain (scale*log2(e) folded in);
 //   * 64-bit offsets throughout (the reference's int32 layer_offset,
 //     mha_kernel.cu:488, overflows on large caches).
 //
 // Tile bookkeeping (T = 16 consecutive positions, r = row in tile, h = head in group):
-//   MFMA A  lane L: row r = L%16, dims (j*4 + L/16)*8 .. +8 for step j = 0..3
-//   MFMA B  lane L: head h = L%16 (zero for h >= group), same dims
-//   MFMA C  lane L: head h = L%16, rows r = 4*(L/16) + i in register i = 0..3
-//   V / O   lane L: rows r = 4*(L/16) + i (load i), dims (L%16)*8 .. +8
-// so the weight of (row 4*(L/16)+i, head h) sits in lane (L/16)*16 + h,
-// register i: the same DPP row as every lane that needs it.
+//   QK  A  lane L: row r = L%16, dims (j*4 + L/16)*8 .. +8 for step j = 0..3
+//   QK  B  lane L: head h = L%16 (zero for h >= group), same dims
+//   QK  C  lane L: head h = L%16, rows r = 4*(L/16) + i in register i = 0..3
+//   V load lane L: rows r = 4*(L/16) + i (load i), columns (L%16)*8 .. +8
+//   PV  A  lane L: head h = L%16, rows 4*(L/16) + i      (= QK C, as bf16)
+//   PV  B  lane L: rows 4*(L/16) + i, column 8*(L%16) + j for product j = 0..7
+//   PV  C  lane L: heads 4*(L/16) + i, column 8*(L%16) + j (accumulator o[j][i])
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
