@@ -87,6 +87,30 @@ __device__ __forceinline__ float row_bcast(float x) {
         float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + SRC, 0xf, 0xf, false));
 }
 
+// x of the lane's DPP partner: quad_perm [1,0,3,2] (0xB1), [2,3,0,1] (0x4E), row_half_mirror (0x141),
+// row_mirror (0x140). Applied in this order with a commutative fold they leave the fold of all 16
+// lanes of a row in every lane, at VALU speed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_partner(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_partner<0xB1>(x));
+    x = fmaxf(x, dpp_partner<0x4E>(x));
+    x = fmaxf(x, dpp_partner<0x141>(x));
+    x = fmaxf(x, dpp_partner<0x140>(x));
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_partner<0xB1>(x);
+    x += dpp_partner<0x4E>(x);
+    x += dpp_partner<0x141>(x);
+    x += dpp_partner<0x140>(x);
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 
@@ -492,41 +516,55 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     __syncthreads();
 
     const bool fused = a.records != nullptr && n_active > 1;
-    const int n_out = a.group * kHeadDim;
-    for (int idx = threadIdx.x; idx < n_out; idx += NW * 64) {
-        const int h = idx >> 7;
-        const int d = idx & (kHeadDim - 1);
+    // One thread per (head, 16-byte column): weights e^(m_w - M) of the waves, weighted sum.
+    const int n_units = a.group * (kHeadDim / 4);
+    const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.ws, 0, (int)((int64_t)a.n_q * a.num_splits * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
+    for (int u = threadIdx.x; u < n_units; u += NW * 64) {
+        const int h = u >> 5;
+        const int c4 = u & 31;
+        float mw[NW];
         float mx = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < NW; ++w) mx = fmaxf(mx, s_m[w][h]);
-        float acc = 0.0f, lsum = 0.0f;
+        for (int w = 0; w < NW; ++w) {
+            mw[w] = s_m[w][h];
+            mx = fmaxf(mx, mw[w]);
+        }
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        float lsum = 0.0f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            const float mw = s_m[w][h];
-            const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - mx);
-            acc += s_o[w][h][d] * f;
+            const float f = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - mx);
+            acc += *reinterpret_cast<const f32x4*>(&s_o[w][h][c4 * 4]) * f;
             lsum += s_l[w][h] * f;
         }
         const int hq = kvh * a.group + h;
         if (n_active == 1) {
-            const float r = acc / lsum;
-            a.out[(int64_t)hq * kHeadDim + d] = f32_to_bf16(r);
-            if (a.out_f32) a.out_f32[(int64_t)hq * kHeadDim + d] = r;
+            f32x4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = acc[e] / lsum;
+            *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
+            if (a.out_f32) {
+                float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
+#pragma unroll
+                for (int e = 0; e < 4; ++e) of[e] = r[e];
+            }
         } else {
             const int64_t S = a.num_splits;
-            float* po = a.ws + ((int64_t)hq * S + split) * kHeadDim + d;
+            const int64_t po = ((int64_t)hq * S + split) * kHeadDim + c4 * 4;  // element offset in the workspace
             if (fused) {
-                // Device-coherent store: it goes past this XCD's L2, so the workgroup
-                // (possibly on another XCD) that does the combine can read it without
+                // Device-coherent store (cache policy sc1): it goes past this XCD's L2, so the
+                // workgroup (possibly on another XCD) that does the combine can read it without
                 // anyone flushing or invalidating a cache.
-                __hip_atomic_store(po, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (d == 0) {
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), part_rsrc,
+                                                       (uint32_t)(po * (int64_t)sizeof(float)), 0, 16);
+                if (c4 == 0) {
                     s_fin[2 * h] = mx;
                     s_fin[2 * h + 1] = lsum;
                 }
             } else {
-                *po = acc;
-                if (d == 0) {
+                *reinterpret_cast<f32x4*>(a.ws + po) = acc;
+                if (c4 == 0) {
                     a.ws[(int64_t)a.n_q * S * kHeadDim + (int64_t)hq * S + split] = mx;
                     a.ws[(int64_t)a.n_q * S * (kHeadDim + 1) + (int64_t)hq * S + split] = lsum;
                 }
@@ -603,8 +641,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) mx = fmaxf(mx, m_reg[j]);
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+        mx = wave_max(mx);
         float den = 0.0f;
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) {
@@ -619,8 +656,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 }
             }
         }
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) den += __shfl_xor(den, d);
+        den = wave_sum(den);
         if (lane == 0) s_den[h] = den;
     }
     if (lane == 0) s_ok[wave] = wave_ok ? 1 : 0;
@@ -638,8 +674,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int NT = NW * 64;
     const int units = a.group * (kHeadDim / 4);
     const int parts = units <= NT ? NT / units : 1;
-    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        a.ws, 0, (int)((int64_t)a.n_q * S * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
     constexpr int kCoherent = 16;  // cache policy: sc1
     for (int u0 = 0; u0 < units; u0 += NT) {
         const int t = u0 + (int)threadIdx.x;
@@ -686,9 +721,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
             const float inv = all_arrived ? 1.0f / s_den[h] : __builtin_nanf("");
             const f32x4 r = acc * inv;
             uint16_t* op = a.out + (int64_t)hq * kHeadDim + c4 * 4;
-            const uint32_t lo = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
-            const uint32_t hi = (uint32_t)f32_to_bf16(r[2]) | ((uint32_t)f32_to_bf16(r[3]) << 16);
-            *reinterpret_cast<uint2*>(op) = make_uint2(lo, hi);
+            *reinterpret_cast<uint2*>(op) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
             if (a.out_f32) {
                 float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
 #pragma unroll
