@@ -604,12 +604,11 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     float* s_den = s_w + G * kMaxSplits;                         // [G] denominators
     int* s_ok = reinterpret_cast<int*>(s_den + G);               // [NW] every record seen
     f32x4* s_part = reinterpret_cast<f32x4*>(s_ok + NW);         // [NW * 64] per-thread partial sums
-    bool wave_ok = true;
-    // One wave per head: wait for the head's records, then M = max m_s, weights
-    // e^(m_s - M), denominator sum l_s * weight -- all from the polled registers.
-    // This workgroup's own (max, sum) comes straight from LDS: its record would be
-    // the last one to become visible.
-    for (int h = wave; h < a.group; h += NW) {
+    // Waits for the records of head h (one wavefront does), then M = max m_s, weights
+    // e^(m_s - M) into the head's row of s_w and the denominator sum l_s * weight -- all from
+    // the polled registers. This workgroup's own (max, sum) comes straight from LDS: its
+    // record would be the last one to become visible. Returns false if a record never came.
+    auto poll_head = [&](int h, float& den_out) -> bool {
         unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         constexpr int kSlots = kMaxSplits / 64;
         float m_reg[kSlots], l_reg[kSlots];
@@ -637,7 +636,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
             if (__all(ok)) break;
             __builtin_amdgcn_s_sleep(2);
         }
-        wave_ok = wave_ok && __all(ok);
+        const bool arrived = __all(ok);
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) mx = fmaxf(mx, m_reg[j]);
@@ -656,7 +655,72 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 }
             }
         }
-        den = wave_sum(den);
+        den_out = wave_sum(den);
+        return arrived;
+    };
+    const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
+    constexpr int kCoherent = 16;  // cache policy: sc1
+
+    if (a.group <= NW) {
+        // One wavefront per head, all the way: poll, then read the head's partials back and write
+        // its 128 outputs, without a workgroup barrier (a wave whose records are in need not wait
+        // for the others). Lane = (16-byte column, half of the splits); the two halves are added
+        // with one xor shuffle. The partials of the other workgroups were acknowledged before
+        // their records were written; they are read with device-coherent 16-byte loads, a
+        // lane's loads all in flight at once.
+        if (wave >= a.group) return;
+        const int h = wave;
+        float den;
+        const bool arrived = poll_head(h, den);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own weights are in LDS
+        __builtin_amdgcn_wave_barrier();
+        const int c4 = lane & 31;
+        const int part = lane >> 5;
+        const int hq = kvh * a.group + h;
+        const uint32_t base = (uint32_t)(((int64_t)hq * S * kHeadDim + c4 * 4) * (int64_t)sizeof(float));
+        const float* w = s_w + h * kMaxSplits;
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        auto gather = [&](auto batch) {
+            constexpr int kBatch = decltype(batch)::value;
+            for (int s0 = part; s0 < SA; s0 += kBatch * 2) {
+                f32x4 v[kBatch];
+                float wv[kBatch];
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const int sp = s0 + j * 2;
+                    const int spc = min(sp, SA - 1);  // in range; the weight below drops the repeat
+                    v[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                         ws_rsrc, base + (uint32_t)spc * (kHeadDim * 4u), 0, kCoherent));
+                    wv[j] = sp < SA ? w[sp] : 0.0f;
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) acc += v[j] * wv[j];
+            }
+        };
+        if (SA <= 16) gather(std::integral_constant<int, 8>{});
+        else gather(std::integral_constant<int, 16>{});
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += __shfl_xor(acc[e], 32);
+        if (part == 0) {
+            // A wait that ran out of patience poisons the output rather than returning a partial sum.
+            const float inv = arrived ? 1.0f / den : __builtin_nanf("");
+            const f32x4 r = acc * inv;
+            *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
+            if (a.out_f32) {
+                float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
+#pragma unroll
+                for (int e = 0; e < 4; ++e) of[e] = r[e];
+            }
+        }
+        return;
+    }
+
+    // More heads than wavefronts: the waves take the heads in turn, then the whole workgroup
+    // shares the read-back.
+    bool wave_ok = true;
+    for (int h = wave; h < a.group; h += NW) {
+        float den;
+        wave_ok = poll_head(h, den) && wave_ok;
         if (lane == 0) s_den[h] = den;
     }
     if (lane == 0) s_ok[wave] = wave_ok ? 1 : 0;
@@ -674,8 +738,6 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int NT = NW * 64;
     const int units = a.group * (kHeadDim / 4);
     const int parts = units <= NT ? NT / units : 1;
-    const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
-    constexpr int kCoherent = 16;  // cache policy: sc1
     for (int u0 = 0; u0 < units; u0 += NT) {
         const int t = u0 + (int)threadIdx.x;
         const int u = t % units;
