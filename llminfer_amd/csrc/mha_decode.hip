@@ -558,7 +558,20 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                 // anyone flushing or invalidating a cache.
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), part_rsrc,
                                                        (uint32_t)(po * (int64_t)sizeof(float)), 0, 16);
-                if (c4 == 0) {
+                if (split != n_active - 1) {
+                    // Publish the head's record as soon as this wavefront's stores are acknowledged:
+                    // the 32 columns of a head are stored by one half of one wavefront, so no
+                    // workgroup barrier is needed.
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    if (c4 == 0) {
+                        unsigned long long* rec = a.records + ((int64_t)hq * S + split) * 2;
+                        const unsigned long long tag = a.epoch & 0xffffffffull;
+                        const unsigned long long m_bits = __builtin_bit_cast(uint32_t, mx);
+                        const unsigned long long l_bits = __builtin_bit_cast(uint32_t, lsum);
+                        __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(rec + 1, tag | (l_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                } else if (c4 == 0) {  // the combiner keeps its own pair in LDS
                     s_fin[2 * h] = mx;
                     s_fin[2 * h + 1] = lsum;
                 }
@@ -576,8 +589,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // ---- fused combine ----
     // The workgroup of the LAST split of this KV head merges the partials of its
     // query heads, so no second launch is needed. Every split publishes, per query
-    // head, a record {epoch | max} {epoch | sum} after its partial outputs have been
-    // acknowledged; the last split's workgroup waits for all records but its own (it
+    // head, a record {epoch | max} {epoch | sum} as soon as the head's partial outputs have
+    // been acknowledged; the last split's workgroup waits for all records but its own (it
     // has its own pair in LDS and its own partials acknowledged). Workgroups are
     // dispatched in index order and the others never wait for anything, so whoever
     // it waits for is already running or done.
@@ -585,20 +598,12 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // uninitialised workspace, an earlier call) reads as "not arrived", so the
     // workspace needs no clearing. The combiner zeroes the records again so that a
     // graph replay of this very call (same epoch) starts clean.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
-    __syncthreads();
     const int S = a.num_splits;  // layout stride of partials and records
     const int SA = n_active;     // splits that hold positions
     const unsigned long long tag = a.epoch & 0xffffffffull;
-    if (split != SA - 1 && threadIdx.x < a.group) {
-        const int h = threadIdx.x;
-        unsigned long long* rec = a.records + ((int64_t)(kvh * a.group + h) * S + split) * 2;
-        const unsigned long long m_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h]);
-        const unsigned long long l_bits = __builtin_bit_cast(uint32_t, s_fin[2 * h + 1]);
-        __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(rec + 1, tag | (l_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (split != SA - 1) return;
+    if (split != SA - 1) return;  // (its records went out above)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the combiner's own partial stores are acknowledged
+    __syncthreads();                                  // ... and its (max, sum) pairs are in LDS
 
     float* s_w = reinterpret_cast<float*>(smem + kCombineBase);  // [G][kMaxSplits] weights
     float* s_den = s_w + G * kMaxSplits;                         // [G] denominators
