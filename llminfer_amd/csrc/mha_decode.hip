@@ -94,21 +94,24 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_partner(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
 }
+__device__ __forceinline__ float row_lane0(float x, int row) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16 * row));
+}
+// Folds over all 64 lanes, the result in every lane: four DPP steps inside the rows, then the four
+// row results are read into scalar registers (no LDS-crossbar shuffles, whose latency adds up).
 __device__ __forceinline__ float wave_max(float x) {
     x = fmaxf(x, dpp_partner<0xB1>(x));
     x = fmaxf(x, dpp_partner<0x4E>(x));
     x = fmaxf(x, dpp_partner<0x141>(x));
     x = fmaxf(x, dpp_partner<0x140>(x));
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
+    return fmaxf(fmaxf(row_lane0(x, 0), row_lane0(x, 1)), fmaxf(row_lane0(x, 2), row_lane0(x, 3)));
 }
 __device__ __forceinline__ float wave_sum(float x) {
     x += dpp_partner<0xB1>(x);
     x += dpp_partner<0x4E>(x);
     x += dpp_partner<0x141>(x);
     x += dpp_partner<0x140>(x);
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
+    return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
