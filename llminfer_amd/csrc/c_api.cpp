@@ -23,10 +23,10 @@ thread_local std::string g_last_error;
 // Context lengths up to this run as one workgroup per KV head; longer ones are
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
-// memory round trips for its combine, while one workgroup of 8 waves streams a
-// whole KV head of 19 tiles in about 7 us: measured at 32 query / 8 KV heads.)
-constexpr int kSinglePassMaxLen8 = 304;  // single pass wins up to here with 8 waves (7.0 vs 7.3 us at 288)
-constexpr int kSinglePassMaxLen4 = 272;  // ... and up to here when only 4 waves are available (7.2 vs 7.3 us)
+// memory round trips for its combine, while one workgroup streams a whole KV
+// head of 13 tiles in about 5.7 us: measured at 32 query / 8 KV heads, single
+// pass 5.5 vs split 5.9 us at 192 positions, 6.3 vs 5.9 us at 224.)
+constexpr int kSinglePassMaxLen = 208;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).
@@ -106,7 +106,7 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
     const size_t per_split_fused = (size_t)a->head_num * (a->head_dim * sizeof(float) + 2 * sizeof(unsigned long long));
 
     const int single_waves_max = (max_waves < wave_cap ? max_waves : wave_cap);  // 8 where the kernel variant allows
-    const int single_pass_max = single_waves_max >= 8 ? kSinglePassMaxLen8 : kSinglePassMaxLen4;
+    const int single_pass_max = kSinglePassMaxLen;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;

@@ -616,9 +616,9 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // e^(m_s - M) into the head's row of s_w and the denominator sum l_s * weight -- all from
     // the polled registers. This workgroup's own (max, sum) comes straight from LDS: its
     // record would be the last one to become visible. Returns false if a record never came.
-    auto poll_head = [&](int h, float& den_out) -> bool {
+    auto poll_head_n = [&](int h, float& den_out, auto slots) -> bool {
         unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
-        constexpr int kSlots = kMaxSplits / 64;
+        constexpr int kSlots = decltype(slots)::value;  // splits per lane
         float m_reg[kSlots], l_reg[kSlots];
         bool ok = false;
         // Bounded wait: every wave leaves this loop even if a record never shows up
@@ -665,6 +665,10 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         }
         den_out = wave_sum(den);
         return arrived;
+    };
+    auto poll_head = [&](int h, float& den_out) -> bool {
+        if (SA <= 64) return poll_head_n(h, den_out, std::integral_constant<int, 1>{});
+        return poll_head_n(h, den_out, std::integral_constant<int, kMaxSplits / 64>{});
     };
     const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
     constexpr int kCoherent = 16;  // cache policy: sc1
