@@ -316,16 +316,16 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // tile read the last valid row and are masked out of the softmax.
     constexpr int kStageBytes = 8192;
     constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
-    // Merge area: NW x G x 128 partial outputs + per-wave and merged (max, sum) pairs.
+    // Epilogue: a wave's G x 128 partial outputs go to the start of its own (drained) ring,
+    // so no wave has to wait for another one's ring. Behind the rings: per-wave and merged
+    // (max, sum) pairs, then the combine area (weights [G][kMaxSplits], denominators [G],
+    // per-wave arrival flags [NW], one 16-byte partial sum per thread).
+    constexpr int kWaveRingBytes = NSTAGE * kStageBytes;
+    static_assert(G * kHeadDim * (int)sizeof(float) <= kWaveRingBytes, "a wave's partial outputs must fit its ring");
     constexpr int kMergeTail = (2 * NW * G + 2 * G) * (int)sizeof(float);
-    constexpr int kMergeBytes = NW * G * kHeadDim * (int)sizeof(float) + kMergeTail;
-    // Combine area (behind the merge area, so the merged (max, sum) pairs stay readable):
-    // weights [G][kMaxSplits], denominators [G], per-wave arrival flags [NW] and one
-    // 16-byte partial sum per thread.
-    constexpr int kCombineBase = (kMergeBytes + 15) & ~15;
+    constexpr int kCombineBase = kRingBytes + ((kMergeTail + 15) & ~15);
     constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float) + NW * 64 * 16;
-    constexpr int kTailBytes = kCombineBase + kCombineBytes;
-    constexpr int kSmemBytes = kRingBytes > kTailBytes ? kRingBytes : kTailBytes;
+    constexpr int kSmemBytes = kCombineBase + kCombineBytes;
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * (NSTAGE * kStageBytes);
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
@@ -494,20 +494,17 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
 
-    // The ring is drained (every tile issued was waited for): reuse its memory
-    // once all waves are done with it.
-    __syncthreads();
-    typedef float (*MergeO)[G][kHeadDim];
+    // This wave's ring is drained (every tile it issued was waited for and read).
     typedef float (*MergeS)[G];
-    MergeO s_o = reinterpret_cast<MergeO>(smem);
-    MergeS s_m = reinterpret_cast<MergeS>(smem + NW * G * kHeadDim * sizeof(float));
+    auto s_o = [&](int w, int h) { return reinterpret_cast<float*>(smem + w * kWaveRingBytes) + h * kHeadDim; };
+    MergeS s_m = reinterpret_cast<MergeS>(smem + kRingBytes);
     MergeS s_l = s_m + NW;
     float* s_fin = reinterpret_cast<float*>(s_l + NW);  // [G][2]: merged (max, sum) per head
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int h = 4 * kg + r;
         if (h < G) {
-            float* dst = &s_o[wave][h][n16 * 8];
+            float* dst = s_o(wave, h) + n16 * 8;
             *reinterpret_cast<f32x4*>(dst) = f32x4{o[0][r], o[1][r], o[2][r], o[3][r]};
             *reinterpret_cast<f32x4*>(dst + 4) = f32x4{o[4][r], o[5][r], o[6][r], o[7][r]};
         }
@@ -538,7 +535,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             const float f = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - mx);
-            acc += *reinterpret_cast<const f32x4*>(&s_o[w][h][c4 * 4]) * f;
+            acc += *reinterpret_cast<const f32x4*>(s_o(w, h) + c4 * 4) * f;
             lsum += s_l[w][h] * f;
         }
         const int hq = kvh * a.group + h;
