@@ -165,3 +165,42 @@ def test_graph_replay_matches_eager(oracle, dev):
         assert torch.equal(out, eager)
         scratch = torch.randn(1 << 16, device=dev).sum().item()  # unrelated eager work between replays
         assert scratch == scratch
+
+
+def test_fused_combine_many_calls_agree_with_the_two_launch_path(dev):
+    """400 back-to-back calls on one workspace, the context, the split count and the query changing from
+    call to call (some enqueued without a synchronisation in between): the fused combine -- whose splits hand
+    their results over through device memory inside one launch -- must give what the split kernel followed by
+    the separate combine kernel gives, up to the rounding of a different summation order."""
+    import torch
+    from llminfer_amd import ops
+    from helpers import from_dev_bf16, to_dev
+    n_q, n_kv, msl = 32, 8, 6000
+    case = synth.make_case(91, ctx=msl, max_seq_len=msl, **QWEN3_4B)
+    k = to_dev(synth.to_head_major(case["k"], n_kv), dev)
+    v = to_dev(synth.to_head_major(case["v"], n_kv), dev)
+    ws = torch.full((ops.workspace_bytes(n_q, 128, msl) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    ws2 = torch.zeros_like(ws)
+    rng = np.random.RandomState(3)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    outs, refs = [], []
+    for it in range(400):
+        ctx = int(rng.choice([209, 300, 777, 1024, 2048, 3001, 4096, 5999]))
+        splits = int(rng.choice([0, 0, 2, 5, 16, 31, 32, 64]))
+        q = torch.randn(n_q * 128, generator=gen, device=dev).to(torch.bfloat16)
+        kw = dict(layer_id=0, pos=ctx - 1, kv_dim=1024, kv_mul=4, head_num=n_q, head_dim=128, max_seq_len=msl,
+                  kv_layout=B.KV_LAYOUT_HEAD_MAJOR, num_splits=splits)
+        out = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        ref = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+        ops.mha_decode(q, k, v, out, ws, force_path=B.PATH_SPLIT_FUSED, **kw)
+        ops.mha_decode(q, k, v, ref, ws2, force_path=B.PATH_SPLIT, **kw)
+        outs.append(out)
+        refs.append(ref)
+        if it % 7 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    for it, (out, ref) in enumerate(zip(outs, refs)):
+        g, r = from_dev_bf16(out), from_dev_bf16(ref)
+        assert np.all(np.isfinite(g)), "call %d" % it
+        assert np.all(np.abs(g - r) <= np.abs(r) / 128 + 1e-6), "call %d: max diff %g" % (it, np.abs(g - r).max())
