@@ -287,6 +287,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--ctx", type=str, default=",".join(map(str, DEFAULT_CTX)))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--dispatch-check", action="store_true",
+                    help="time the automatic plan against forced single-pass / split plans at every --ctx")
     ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
     ap.add_argument("--heads", type=int, default=N_Q, help="query heads (32 = Qwen3-4B, 64 = Qwen3-32B head layout)")
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
@@ -328,30 +330,30 @@ def main():
     ws = torch.empty(ops.workspace_bytes(n_q, HEAD_DIM, max(ctx_list)) // 4, dtype=torch.float32, device=dev)
     esz = 2
 
-    def call_args(ctx, s):
+    def call_args(ctx, s, **over):
         off = regions[(ctx, s)] * esz
         return ops.make_mha_args(q, k.data_ptr() + off, v.data_ptr() + off, out, ws, layer_id=0, pos=ctx - 1,
                                  kv_dim=KV_DIM, kv_mul=n_q // N_KV, head_num=n_q, head_dim=HEAD_DIM,
-                                 max_seq_len=ctx, kv_layout=args.layout)
+                                 max_seq_len=ctx, kv_layout=args.layout, **over)
 
     plans = {ctx: ops.mha_plan(call_args(ctx, 0)) for ctx in ctx_list}
     stream = torch.cuda.Stream()
     decode = B.lib().llmi_hip_mha_decode
 
-    def enqueue(ctxs, steps):
+    def enqueue(ctxs, steps, **over):
         for s in range(steps):
             for ctx in ctxs:
-                a = call_args(ctx, s % SLICES)
+                a = call_args(ctx, s % SLICES, **over)
                 a.stream = stream.cuda_stream
                 B.check(decode(ctypes.byref(a)), "llmi_hip_mha_decode")
 
-    def capture(ctxs):
+    def capture(ctxs, **over):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
-            enqueue(ctxs, 1)  # eager once: loads the code objects before capture
+            enqueue(ctxs, 1, **over)  # eager once: loads the code objects before capture
             stream.synchronize()
             with torch.cuda.graph(g, stream=stream):
-                enqueue(ctxs, SLICES)
+                enqueue(ctxs, SLICES, **over)
         return g
 
     def time_graph(g, replays):
@@ -364,6 +366,38 @@ def main():
             e1.record(stream)
         e1.synchronize()
         return e0.elapsed_time(e1)  # ms
+
+    if args.dispatch_check:
+        # What the dispatcher picks against forced alternatives, per context length: single pass, and the
+        # fused split path at several split counts (4 waves); same timing method as the per-context figures.
+        rows = []
+        for ctx in ctx_list:
+            def timed(**over):
+                g = capture([ctx], **over)
+                time_graph(g, 2)
+                torch.cuda.synchronize()
+                n = max(SLICES, args.steps // 4 // SLICES * SLICES)
+                t = time_graph(g, n // SLICES)
+                torch.cuda.synchronize()
+                return t * 1e3 / n
+            auto = timed()
+            alts = {}
+            if ctx <= 1024:
+                alts["single"] = timed(force_path=B.PATH_SINGLE_PASS)
+            tiles = (ctx + 15) // 16
+            for sp in (4, 8, 16, 32, 64):
+                if sp <= tiles:
+                    alts["split%d" % sp] = timed(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
+            best = min(alts, key=alts.get)
+            p = plans[ctx]
+            rows.append({"ctx": ctx, "auto_us": round(auto, 2), "auto_plan": "path%d S=%d W=%d" % (p.path, p.num_splits, p.waves_per_group),
+                         "best_forced": best, "best_forced_us": round(alts[best], 2),
+                         "auto_over_best": round(auto / alts[best], 3),
+                         "forced_us": {k2: round(v2, 2) for k2, v2 in alts.items()}})
+        print(json.dumps({"metric": "dispatch check: auto plan against forced paths, us per layer call", "n_gpus": 1,
+                          "config": {"workload": "%d Q / 8 KV heads, %s layout" % (n_q, "head-major" if args.layout == 1 else "position-major")},
+                          "rows": rows, "worst_auto_over_best": max(r["auto_over_best"] for r in rows)}))
+        return 0
 
     # ---- the timed region: K steps of the whole sweep ----------------------
     steps = max(SLICES, (args.steps + SLICES - 1) // SLICES * SLICES)

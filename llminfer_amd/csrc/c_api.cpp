@@ -24,9 +24,9 @@ thread_local std::string g_last_error;
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
 // memory round trips for its combine, while one workgroup streams a whole KV
-// head of 13 tiles in about 5.7 us: measured at 32 query / 8 KV heads, single
-// pass 5.5 vs split 5.9 us at 192 positions, 6.3 vs 5.9 us at 224.)
-constexpr int kSinglePassMaxLen = 208;
+// head of 10 tiles in about 5.2 us: measured at 32 query / 8 KV heads under graph
+// replay, single pass 5.2 vs split 5.9 us at 160 positions, 6.3 vs 6.0 us at 176.)
+constexpr int kSinglePassMaxLen = 160;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).

@@ -57,7 +57,7 @@ def test_split_sweep_matches_oracle(oracle, dev, splits, waves, path):
     _check(oracle, dev, case, num_splits=splits, waves_per_group=waves, force_path=path)
 
 
-@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 207, 208, 209, 255, 256, 257, 1000, 4097])
+@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 159, 160, 161, 255, 256, 257, 1000, 4097])
 @pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT, B.PATH_SPLIT_FUSED])
 def test_ragged_lengths(oracle, dev, ctx, path):
     """Lengths around the 16-row tile, the wave count and the dispatch threshold; the cache rows past
