@@ -374,12 +374,17 @@ def main():
         for ctx in ctx_list:
             def timed(**over):
                 g = capture([ctx], **over)
-                time_graph(g, 2)
+                time_graph(g, 8)
                 torch.cuda.synchronize()
                 n = max(SLICES, args.steps // 4 // SLICES * SLICES)
-                t = time_graph(g, n // SLICES)
-                torch.cuda.synchronize()
-                return t * 1e3 / n
+                best_ms = None
+                for _ in range(3):  # best of three batches: a batch now and then runs 1-2 us per call slow
+                    t = time_graph(g, n // SLICES)
+                    torch.cuda.synchronize()
+                    best_ms = t if best_ms is None else min(best_ms, t)
+                return best_ms * 1e3 / n
+            if not rows:
+                timed()  # the first graph timed in a process runs 1-2 us per call slow: discard one
             auto = timed()
             alts = {}
             if ctx <= 1024:

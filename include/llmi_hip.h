@@ -104,7 +104,8 @@ typedef struct llmi_mha_args {
 typedef struct llmi_mha_plan {
     int32_t path;             /* LLMI_PATH_SINGLE_PASS, LLMI_PATH_SPLIT or LLMI_PATH_SPLIT_FUSED */
     int32_t num_splits;       /* 1 for single-pass                                       */
-    int32_t rows_per_split;   /* multiple of 16                                          */
+    int32_t rows_per_split;   /* most positions one split handles (multiple of 16): a head's 16-position
+                                 tiles go to the splits in contiguous runs that differ by at most one tile */
     int32_t waves_per_group;
     int32_t group_pad;        /* query heads per KV head rounded up to 1,2,4,8,16        */
     size_t workspace_needed;  /* bytes of workspace this plan uses (0 for single-pass)   */

@@ -145,11 +145,11 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
             if (cap < 2) return LLMI_ERR_WORKSPACE;
             if ((size_t)want > cap) want = (int)cap;
-            tiles_per_split = ceil_div(tiles, want);
-        } else {
-            tiles_per_split = ceil_div(tiles, want);
         }
-        num_splits = ceil_div(tiles, tiles_per_split);  // no empty splits
+        // The kernel deals the tiles to the splits in contiguous runs that differ by at most one
+        // tile, so no split is empty as long as there are no more splits than tiles.
+        num_splits = want < tiles ? want : tiles;
+        tiles_per_split = ceil_div(tiles, num_splits);
         if (num_splits > 1) {
             const size_t need = (fused ? per_split_fused : per_split_plain) * (size_t)num_splits + (fused ? 16 : 0);
             if (!a->workspace || a->workspace_bytes < need) return LLMI_ERR_WORKSPACE;

@@ -184,7 +184,6 @@ struct KernelArgs {
     int32_t group;        // query heads per KV head
     int32_t n_q;          // query heads
     int32_t num_splits;
-    int32_t rows_per_split;  // multiple of kTile
     float scale_log2e;       // log2(e) / sqrt(head_dim)
     // Fused append (APPEND kernels only): q is the raw query; the new token's K
     // row is normalised + rotated, its V row copied, both stored at position
@@ -266,22 +265,25 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
 
-    // Static launch: the host never makes empty splits. With a position read from
-    // device memory the grid was sized for the largest position; the same rule as the
-    // host's (equal tile counts, no empty split in the middle) is applied here, and the
-    // workgroups beyond the last active split leave at once.
-    int seq_len = a.seq_len, rows_per_split = a.rows_per_split, n_active = a.num_splits;
+    // A KV head's 16-position tiles are dealt to the splits in contiguous runs whose lengths
+    // differ by at most one tile (the first tiles % S splits get the longer run), so every split
+    // has work whenever there are at least S tiles and the last split -- the one that merges,
+    // and in the append variant the one that holds the new token -- never has the longest run.
+    // With a position read from device memory the grid was sized for the largest position:
+    // the same rule is applied to the tiles there are, and splits beyond the tile count leave
+    // at once.
+    int seq_len = a.seq_len, n_active = a.num_splits;
     if constexpr (DYN) {
         seq_len = max(0, min(*a.pos_dev, a.seq_len - 1)) + 1;
-        const int tiles = (seq_len + kTile - 1) / kTile;
-        const int tps = (tiles + a.num_splits - 1) / a.num_splits;
-        rows_per_split = tps * kTile;
-        n_active = (tiles + tps - 1) / tps;
+        n_active = min(a.num_splits, (seq_len + kTile - 1) / kTile);
         if (split >= n_active) return;
     }
-    const int begin = split * rows_per_split;
-    const int nrows = min(rows_per_split, seq_len - begin);  // > 0
-    const int ntiles = (nrows + kTile - 1) / kTile;
+    const int total_tiles = (seq_len + kTile - 1) / kTile;
+    const int run = total_tiles / n_active;     // >= 1: the host never asks for more splits than tiles
+    const int longer = total_tiles % n_active;  // splits 0 .. longer-1 take run + 1 tiles
+    const int ntiles = run + (split < longer ? 1 : 0);
+    const int begin = (split * run + min(split, longer)) * kTile;
+    const int nrows = min(ntiles * kTile, seq_len - begin);  // > 0
 
     // Filled in below, once the first tiles are on their way.
     u32x4 qb[4];                       // query group, MFMA B operand
@@ -918,7 +920,6 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
     ka.group = args.kv_mul;
     ka.n_q = args.head_num;
     ka.num_splits = plan.num_splits;
-    ka.rows_per_split = plan.rows_per_split;
     ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
     if (append) {
         ka.k_new = static_cast<const uint16_t*>(append->key_new);

@@ -118,7 +118,8 @@ def test_plan_long_context_splits_without_empty_splits(ctx):
     rc, p = plan(good_args(pos=ctx - 1, max_seq_len=ctx))
     assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and 2 <= p.num_splits <= 256
     assert p.rows_per_split % 16 == 0
-    assert (p.num_splits - 1) * p.rows_per_split < ctx <= p.num_splits * p.rows_per_split
+    tiles = (ctx + 15) // 16
+    assert p.num_splits <= tiles and p.rows_per_split == -(-tiles // p.num_splits) * 16  # no split without a tile
     assert p.workspace_needed <= B.lib().llmi_hip_mha_workspace_bytes(32, 128, ctx)
     assert p.group_pad == 4 and p.waves_per_group in (1, 2, 4, 8)
 
@@ -126,8 +127,8 @@ def test_plan_long_context_splits_without_empty_splits(ctx):
 def test_plan_honours_requests_and_clamps_to_the_workspace():
     rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=16))
     assert rc == 0 and p.path == B.PATH_SPLIT and p.num_splits == 16 and p.rows_per_split == 256
-    rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=200))  # 256 tiles / 200 -> 2 tiles per split
-    assert rc == 0 and p.num_splits == 128
+    rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=200))  # 256 tiles: 56 splits of 2, 144 of 1
+    assert rc == 0 and p.num_splits == 200 and p.rows_per_split == 32
     rc, p = plan(good_args(force_path=B.PATH_SINGLE_PASS))
     assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1
     # a reference-sized workspace [head_num, 4*max_seq_len] fp32 (qwen3_fused.cpp:502) limits the auto split count
