@@ -127,11 +127,10 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
         waves = a->waves_per_group ? a->waves_per_group : auto_waves;
         int want = a->num_splits;
         if (want == 0) {
-            // Auto: a few workgroups per CU, at least one tile per wave, and
-            // no more splits than the caller's workspace can hold.
-            // One workgroup per CU for long contexts; for short ones one tile per
+            // Auto: one workgroup per CU for long contexts; for short ones one tile per
             // wave, but never fewer than kMinGroups workgroups (idle waves cost less
-            // than idle CUs: measured at ctx 256..2048).
+            // than idle CUs: measured at ctx 256..2048); and no more splits than the
+            // caller's workspace can hold.
             int target = kTargetGroups / n_kv;
             if (target < 2) target = 2;
             if (target > kMaxSplits) target = kMaxSplits;
