@@ -427,16 +427,16 @@ def main():
         t = time_graph(g, n // SLICES)
         torch.cuda.synchronize()
         us = t * 1e3 / n
-        # Spread: 32 batches of two replays each, an event between batches, nothing else on the stream.
+        # Spread: 32 batches of eight replays each, an event between batches, nothing else on the stream.
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(33)]
         with torch.cuda.stream(stream):
             marks[0].record(stream)
             for b in range(32):
-                g.replay()
-                g.replay()
+                for _ in range(8):
+                    g.replay()
                 marks[b + 1].record(stream)
         marks[-1].synchronize()
-        batch_us = sorted(marks[b].elapsed_time(marks[b + 1]) * 1e3 / (2 * SLICES) for b in range(32))
+        batch_us = sorted(marks[b].elapsed_time(marks[b + 1]) * 1e3 / (8 * SLICES) for b in range(32))
         gbs = algorithmic_bytes(ctx, n_q) / (us * 1e-6) / 1e9
         p = plans[ctx]
         per_ctx.append({"ctx": ctx, "us_per_layer": round(us, 3), "us_p10": round(batch_us[3], 3),
