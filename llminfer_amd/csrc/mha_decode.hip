@@ -181,6 +181,7 @@ struct KernelArgs {
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
+    bool stagger;                  // walk the tiles of a split from a split-dependent starting point (plain variant only)
     int32_t group;        // query heads per KV head
     int32_t n_q;          // query heads
     int32_t num_splits;
@@ -256,7 +257,7 @@ __device__ __forceinline__ void norm_rope_row(const uint16_t* row, const uint16_
     }
 }
 
-template <int G, int NW, int NSTAGE, bool APPEND, bool DYN>
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
 __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
@@ -418,9 +419,22 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
 
     // Wave w owns tiles w, w+NW, ...: NSTAGE of them are always in flight.
     const int n_my = wave < ntiles ? (ntiles - wave + NW - 1) / NW : 0;
+    // STAGGER (position-major layout): the splits of a head walk their tiles from different starting
+    // points (split s starts s mod 4 tiles into its wave's sequence and wraps round), so that
+    // workgroups running in step do not all sit at the same offset of their runs. At 8192 positions
+    // the runs start exactly 512 KiB apart and walking them in step costs 1.7 us of 13.6. The
+    // head-major layout gains nothing from it and the bookkeeping costs 0.08 us per call, so it
+    // is compiled in only where it is used.
+    const int rot = STAGGER ? min(split & 3, max(n_my - 1, 0)) : 0;
+    auto tile_of = [&](int i) {
+        if constexpr (!STAGGER) return wave + i * NW;
+        int ii = i + rot;
+        if (ii >= n_my) ii -= n_my;
+        return wave + ii * NW;
+    };
 #pragma unroll
     for (int s0 = 0; s0 < NSTAGE; ++s0)
-        if (s0 < n_my) issue_tile(wave + s0 * NW, s0);
+        if (s0 < n_my) issue_tile(tile_of(s0), s0);
     // (The first tiles are already on their way: the query's own loads, and in the
     // append variant its normalisation, overlap with them.)
     // Query group as the MFMA B operand (zero columns beyond the group). The
@@ -465,7 +479,7 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         wait_tiles_in_flight(min(NSTAGE - 1, n_my - 1 - i));
         read_tile(stage, r);
         if constexpr (APPEND) {
-            const int t = wave + i * NW;
+            const int t = tile_of(i);
             if (holds_new_row && t == ntiles - 1) {
                 // Row `fresh` of this tile is the new token; the rows after it are
                 // clamped re-reads of its (still unwritten) cache slot: give them
@@ -485,8 +499,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
                                               kvh * a.slot_head_stride + n16 * 8) = v_fresh;
             }
         }
-        if (i + NSTAGE < n_my) issue_tile(wave + (i + NSTAGE) * NW, stage);
-        compute_tile(wave + i * NW, r);
+        if (i + NSTAGE < n_my) issue_tile(tile_of(i + NSTAGE), stage);
+        compute_tile(tile_of(i), r);
         stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
     }
 
@@ -868,6 +882,8 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
         }
     } else {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else if (ka.stagger && ka.num_splits > 1)
+            hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false>), grid, dim3(NW * 64), 0, stream, ka);
     }
 }
@@ -917,6 +933,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
     }
     ka.seq_len = args.pos + 1;
+    ka.stagger = args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR;
     ka.group = args.kv_mul;
     ka.n_q = args.head_num;
     ka.num_splits = plan.num_splits;
