@@ -271,6 +271,14 @@ int llmi_hip_qkv_gemv(const llmi_qkv_gemv_args* args);
 
 /* ---- misc ---------------------------------------------------------------- */
 int llmi_hip_abi_version(void);
+/* No counterpart in the reference (its combine is a second launch and waits for nothing). In the fused
+ * split path the workgroup that merges a KV head's partial results polls device memory until every other
+ * split of the head has published its record. That wait is bounded: after `polls` unsuccessful polls
+ * (default 4194304, seconds of wall time, which only a fault elsewhere on the GPU can reach) it stops and
+ * writes NaN to the outputs of its heads instead of hanging the device. Applies to launches enqueued
+ * after the call; returns the previous limit. 0 makes every fused launch give up at once: the way to
+ * exercise the failure path in a test. */
+int32_t llmi_hip_set_poll_limit(int32_t polls);
 const char* llmi_hip_strerror(int status);
 /* The last HIP error string seen by this library on the calling thread ("" if none). */
 const char* llmi_hip_last_error(void);

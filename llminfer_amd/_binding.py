@@ -109,6 +109,7 @@ SYMBOLS = {
     "llmi_hip_memcpy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_void_p, c_i32]),
     "llmi_hip_memset_zero": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, c_i32]),
     "llmi_hip_abi_version": (ctypes.c_int, []),
+    "llmi_hip_set_poll_limit": (c_i32, [c_i32]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
 }

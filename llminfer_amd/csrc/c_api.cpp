@@ -66,6 +66,10 @@ unsigned long long next_epoch() {
     return e;
 }
 
+// Default: far beyond any real kernel time (seconds), yet finite.
+static std::atomic<int> g_poll_limit{1 << 22};
+int poll_limit() { return g_poll_limit.load(std::memory_order_relaxed); }
+
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
 
 static int validate_mha(const llmi_mha_args* a) {
@@ -358,6 +362,10 @@ int llmi_hip_qkv_gemv(const llmi_qkv_gemv_args* a) {
 }
 
 int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }
+
+int32_t llmi_hip_set_poll_limit(int32_t polls) {
+    return llmi::g_poll_limit.exchange(polls < 0 ? 0 : polls, std::memory_order_relaxed);
+}
 
 const char* llmi_hip_strerror(int status) {
     switch (status) {

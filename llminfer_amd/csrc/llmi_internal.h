@@ -20,6 +20,8 @@ int check_launch();
 
 // A fresh 48-bit tag per decode call (never 0), for the arrival cells of the fused combine.
 unsigned long long next_epoch();
+// Polls (each followed by a short sleep) the fused combine waits for the other splits.
+int poll_limit();
 
 // `append` non-null: the fused QK-Norm + RoPE + K/V append variant.
 int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append = nullptr);

@@ -59,10 +59,6 @@ namespace {
 
 constexpr int kTile = 16;      // positions per MFMA tile
 constexpr int kHeadDim = 128;
-// Polls (each followed by a short sleep) the fused combine waits for the other splits: far
-// beyond any real kernel time, yet finite.
-constexpr int kMaxSpins = 1 << 22;
-
 // Build-time tuning knobs.
 #ifndef LLMI_NT_LOADS
 #define LLMI_NT_LOADS 1  // K/V are read once: stream them past the caches
@@ -181,6 +177,7 @@ struct KernelArgs {
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
+    int32_t max_polls;             // polls of the fused combine before it gives up and writes NaN
     bool stagger;                  // walk the tiles of a split from a split-dependent starting point (plain variant only)
     int32_t group;        // query heads per KV head
     int32_t n_q;          // query heads
@@ -633,10 +630,15 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         constexpr int kSlots = decltype(slots)::value;  // splits per lane
         float m_reg[kSlots], l_reg[kSlots];
+#pragma unroll
+        for (int j = 0; j < kSlots; ++j) {
+            m_reg[j] = -INFINITY;
+            l_reg[j] = 0.0f;
+        }
         bool ok = false;
         // Bounded wait: every wave leaves this loop even if a record never shows up
         // (the result is then poisoned below instead of hanging the GPU).
-        for (int spin = 0; spin < kMaxSpins; ++spin) {
+        for (int spin = 0; spin < a.max_polls; ++spin) {
             ok = true;
 #pragma unroll
             for (int j = 0; j < kSlots; ++j) {
@@ -933,6 +935,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
     }
     ka.seq_len = args.pos + 1;
+    ka.max_polls = poll_limit();
     ka.stagger = args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR;
     ka.group = args.kv_mul;
     ka.n_q = args.head_num;

@@ -218,3 +218,12 @@ def test_gemv_argument_checks():
         b = B.QkvGemvArgs.from_buffer_copy(q)
         setattr(b, field, value)
         assert L.llmi_hip_qkv_gemv(ctypes.byref(b)) == B.STATUS[status], field
+
+
+def test_poll_limit_round_trip():
+    """The bound on the fused combine's wait: default 2^22 polls, negative values clamp to zero,
+    the setter returns what was there before (no GPU involved)."""
+    lib = B.lib()
+    assert lib.llmi_hip_set_poll_limit(7) == 1 << 22
+    assert lib.llmi_hip_set_poll_limit(-5) == 7
+    assert lib.llmi_hip_set_poll_limit(1 << 22) == 0

@@ -204,3 +204,21 @@ def test_fused_combine_many_calls_agree_with_the_two_launch_path(dev):
         g, r = from_dev_bf16(out), from_dev_bf16(ref)
         assert np.all(np.isfinite(g)), "call %d" % it
         assert np.all(np.abs(g - r) <= np.abs(r) / 128 + 1e-6), "call %d: max diff %g" % (it, np.abs(g - r).max())
+
+
+@pytest.mark.parametrize("kv_mul,n_kv", [(4, 8), (16, 2)])
+def test_fused_combine_gives_up_with_nan_instead_of_hanging(oracle, dev, kv_mul, n_kv):
+    """The merging workgroup's wait for the other splits is bounded. With the limit forced to zero
+    polls from the host every fused launch gives up at once: the kernel still ends normally and
+    every output is NaN (never a plausible wrong number). With the limit restored the same call
+    on the same data gives the oracle's answer. Both merge variants (one wavefront per head, and
+    heads shared out when a group has more heads than the workgroup has wavefronts)."""
+    case = synth.make_case(31, ctx=1000, n_q=kv_mul * n_kv, n_kv=n_kv)
+    prev = B.lib().llmi_hip_set_poll_limit(0)
+    try:
+        assert prev == 1 << 22
+        got16, got32 = run_hip(case, dev, force_path=B.PATH_SPLIT_FUSED, num_splits=8)
+    finally:
+        assert B.lib().llmi_hip_set_poll_limit(prev) == 0
+    assert np.all(np.isnan(got16)) and np.all(np.isnan(got32))
+    _check(oracle, dev, case, force_path=B.PATH_SPLIT_FUSED, num_splits=8)
