@@ -151,6 +151,14 @@ __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t 
 #endif
 }
 
+// Same, with a full 64-bit address per lane and without the streaming hint: for small
+// operands that many workgroups share (they stay in L2).
+__device__ __forceinline__ void dma16_gather(const void* ptr, uint32_t lds_off) {
+    const uint32_t slds = (uint32_t)__builtin_amdgcn_readfirstlane(lds_off);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(slds), "v"(ptr) : "memory");
+}
+
 // Waits until at most `newer_tiles` whole tiles (8 loads each) are still in flight.
 __device__ __forceinline__ void wait_tiles_in_flight(int newer_tiles) {
     if (newer_tiles <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -195,63 +203,50 @@ struct KernelArgs {
     float eps;
 };
 
-// RMSNorm * weight + half-rotation RoPE of one 128-wide row, for the lane's 32
-// elements in the MFMA operand layout (dims (j*4+kg)*8 .. +8, j = 0..3), rounded
-// to bf16. The four lanes that share a row (kg = 0..3 of one DPP column) add up
-// the sum of squares with two xor shuffles. Same chain as the stand-alone kernel
-// (x*w*r, then a*cos - b*sin / a*sin + b*cos on the pairs (i, i+64)).
-__device__ __forceinline__ void norm_rope_row(const uint16_t* row, const uint16_t* w, const float* sin_row,
-                                              const float* cos_row, float eps, int kg, u32x4 (&out)[4]) {
-    float x[4][8], wt[4][8];
+// RMSNorm * weight + half-rotation RoPE of 128-wide bf16 rows held in LDS, in place, by one
+// wavefront: the 16 lanes of DPP row r take row `row` of `rows` (256 bytes each); lane p of them
+// takes elements 4*(p&1) .. +3 of 16-byte chunk p>>1 and of its rotary partner, chunk (p>>1) + 8,
+// so a lane touches 8 elements, reads only what it overwrites, and the sum of squares is one
+// DPP row fold. `w`: the 256-byte norm weights; `sin16` / `cos16`: the 64 sines / cosines of the
+// position (lane p needs exactly 16-byte chunk p of each). Same chain as the stand-alone kernel
+// (x*w*r, then a*cos - b*sin / a*sin + b*cos on the pairs (i, i+64)), rounded to bf16 once.
+__device__ __forceinline__ void norm_rope_rows_lds(char* rows, const char* w, const char* sin16, const char* cos16,
+                                                   int row, int p, float eps) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const int c = p >> 1, hf = p & 1;
+    u32x2* lo_p = reinterpret_cast<u32x2*>(rows + (row * 16 + c) * 16 + hf * 8);
+    u32x2* hi_p = reinterpret_cast<u32x2*>(rows + (row * 16 + c + 8) * 16 + hf * 8);
+    const u32x2 xl = *lo_p, xh = *hi_p;
+    const u32x2 wl = *reinterpret_cast<const u32x2*>(w + c * 16 + hf * 8);
+    const u32x2 wh = *reinterpret_cast<const u32x2*>(w + (c + 8) * 16 + hf * 8);
+    const f32x4 sn = *reinterpret_cast<const f32x4*>(sin16 + p * 16);
+    const f32x4 cs = *reinterpret_cast<const f32x4*>(cos16 + p * 16);
+    const uint32_t xl0 = xl[0], xl1 = xl[1], xh0 = xh[0], xh1 = xh[1];
+    const uint32_t wl0 = wl[0], wl1 = wl[1], wh0 = wh[0], wh1 = wh[1];
+    const float a[4] = {bf16_lo(xl0), bf16_hi(xl0), bf16_lo(xl1), bf16_hi(xl1)};
+    const float b[4] = {bf16_lo(xh0), bf16_hi(xh0), bf16_lo(xh1), bf16_hi(xh1)};
+    const float wa[4] = {bf16_lo(wl0), bf16_hi(wl0), bf16_lo(wl1), bf16_hi(wl1)};
+    const float wb[4] = {bf16_lo(wh0), bf16_hi(wh0), bf16_lo(wh1), bf16_hi(wh1)};
     float ss = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const u32x4 xr = *reinterpret_cast<const u32x4*>(row + (j * 4 + kg) * 8);
-        const u32x4 wr = *reinterpret_cast<const u32x4*>(w + (j * 4 + kg) * 8);
+    for (int e = 0; e < 4; ++e) ss += a[e] * a[e];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            x[j][2 * c] = bf16_lo(xr[c]);
-            x[j][2 * c + 1] = bf16_hi(xr[c]);
-            wt[j][2 * c] = bf16_lo(wr[c]);
-            wt[j][2 * c + 1] = bf16_hi(wr[c]);
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
-    }
-    ss += __shfl_xor(ss, 16);
-    ss += __shfl_xor(ss, 32);
+    for (int e = 0; e < 4; ++e) ss += b[e] * b[e];
+    ss += dpp_partner<0xB1>(ss);
+    ss += dpp_partner<0x4E>(ss);
+    ss += dpp_partner<0x141>(ss);
+    ss += dpp_partner<0x140>(ss);
     const float r = 1.0f / sqrtf(ss / (float)kHeadDim + eps);
+    float ol[4], oh[4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        float sn[8], cs[8];
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const f32x4 s4 = *reinterpret_cast<const f32x4*>(sin_row + (j * 4 + kg) * 8 + 4 * c);
-            const f32x4 c4 = *reinterpret_cast<const f32x4*>(cos_row + (j * 4 + kg) * 8 + 4 * c);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                sn[4 * c + e] = s4[e];
-                cs[4 * c + e] = c4[e];
-            }
-        }
-        uint32_t lo[4], hi[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            uint32_t pl = 0, ph = 0;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int e = 2 * c + half;
-                const float av = x[j][e] * wt[j][e] * r;
-                const float bv = x[j + 2][e] * wt[j + 2][e] * r;
-                pl |= (uint32_t)f32_to_bf16(av * cs[e] - bv * sn[e]) << (16 * half);
-                ph |= (uint32_t)f32_to_bf16(av * sn[e] + bv * cs[e]) << (16 * half);
-            }
-            lo[c] = pl;
-            hi[c] = ph;
-        }
-        out[j] = u32x4{lo[0], lo[1], lo[2], lo[3]};
-        out[j + 2] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    for (int e = 0; e < 4; ++e) {
+        const float av = a[e] * wa[e] * r;
+        const float bv = b[e] * wb[e] * r;
+        ol[e] = av * cs[e] - bv * sn[e];
+        oh[e] = av * sn[e] + bv * cs[e];
     }
+    *lo_p = u32x2{pack_bf16(ol[0], ol[1]), pack_bf16(ol[2], ol[3])};
+    *hi_p = u32x2{pack_bf16(oh[0], oh[1]), pack_bf16(oh[2], oh[3])};
 }
 
 template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
@@ -287,7 +282,8 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     u32x4 qb[4];                       // query group, MFMA B operand
     u32x4 k_fresh[4] = {};             // append variant: the new token's K row (operand layout) ...
     u32x4 v_fresh = {0u, 0u, 0u, 0u};  // ... and V row chunk
-    const bool holds_new_row = APPEND && split == n_active - 1;
+    // Append variant: the wave that owns the last tile of the last split holds the new token.
+    const bool holds_new_row = APPEND && split == n_active - 1 && ((ntiles - 1) & (NW - 1)) == wave;
 
     // Wave-uniform 64-bit bases of this split; lanes add 32-bit byte offsets
     // (scalar-base + vector-offset addressing, no 64-bit multiplies per load).
@@ -325,7 +321,15 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int kMergeTail = (2 * NW * G + 2 * G) * (int)sizeof(float);
     constexpr int kCombineBase = kRingBytes + ((kMergeTail + 15) & ~15);
     constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float) + NW * 64 * 16;
-    constexpr int kSmemBytes = kCombineBase + kCombineBytes;
+    // Per wave, 1 KiB LDS-DMA slots for the small operands: the query rows of the group (16 chunks
+    // of 16 bytes per head, four heads to a slot) and, in the append variant in front of them, the
+    // operands of the fused QK-Norm + RoPE (slot 0: q_norm | k_norm | sin row | cos row, 16 chunks
+    // each; slot 1: new K row | new V row).
+    constexpr int kQSlots = (G * 16 + 63) / 64;
+    constexpr int kQOff = APPEND ? 2048 : 0;
+    constexpr int kStageSlots = kQSlots + (APPEND ? 2 : 0);
+    constexpr int kStagingBase = (kCombineBase + kCombineBytes + 1023) & ~1023;
+    constexpr int kSmemBytes = kStagingBase + NW * kStageSlots * 1024;
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * (NSTAGE * kStageBytes);
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
@@ -429,46 +433,69 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
         if (ii >= n_my) ii -= n_my;
         return wave + ii * NW;
     };
+    // The query rows (and in the append variant the operands of the fused QK-Norm + RoPE) go to
+    // LDS by DMA *ahead of* the first K/V tiles. Loads complete in order, so they are there
+    // after one memory round trip: the normalisation runs while the tiles are still in flight,
+    // and the first tile is worked on as soon as it lands. As ordinary loads their wait would be
+    // placed by the compiler, which does not know about the DMA loads: it would also wait for
+    // every tile issued before that point.
+    char* my_staging = smem + kStagingBase + wave * (kStageSlots * 1024);
+    {
+        const uint32_t st = (uint32_t)(uintptr_t)my_staging;
+        const int c16 = lane & 15, which = lane >> 4;
+        if constexpr (APPEND) {
+            const float* sin_row = a.sin_cache + (int64_t)(seq_len - 1) * 64;
+            const float* cos_row = a.cos_cache + (int64_t)(seq_len - 1) * 64;
+            const void* p0 = which == 0   ? static_cast<const void*>(a.norm_w + c16 * 8)
+                             : which == 1 ? static_cast<const void*>(a.norm_w + kHeadDim + c16 * 8)
+                             : which == 2 ? static_cast<const void*>(sin_row + c16 * 4)
+                                          : static_cast<const void*>(cos_row + c16 * 4);
+            dma16_gather(p0, st);
+            if (holds_new_row) {
+                const void* p1 = (which & 1) == 0 ? static_cast<const void*>(a.k_new + kvh * kHeadDim + c16 * 8)
+                                                  : static_cast<const void*>(a.v_new + kvh * kHeadDim + c16 * 8);
+                dma16_gather(p1, st + 1024);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kQSlots; ++i) {
+            const int head = min(which + 4 * i, a.group - 1);  // chunk lane + 64*i: head (lane + 64*i) / 16
+            dma16_gather(a.q + (int64_t)(kvh * a.group + head) * kHeadDim + c16 * 8, st + kQOff + i * 1024);
+        }
+    }
 #pragma unroll
     for (int s0 = 0; s0 < NSTAGE; ++s0)
         if (s0 < n_my) issue_tile(tile_of(s0), s0);
-    // (The first tiles are already on their way: the query's own loads, and in the
-    // append variant its normalisation, overlap with them.)
-    // Query group as the MFMA B operand (zero columns beyond the group). The
-    // load itself is unpredicated (padding lanes re-read the last head) so
-    // that it does not force a full wait on the first K/V tile.
+    // Query group as the MFMA B operand (zero columns beyond the group; rows beyond it
+    // were filled with copies of its last row).
     {
-        const int hq = kvh * a.group + min(n16, a.group - 1);
-        const uint16_t* qp = a.q + (int64_t)hq * kHeadDim;
-        const bool live = n16 < a.group;
+        // Everything issued before the tiles has landed once only the tiles are in flight.
+        wait_tiles_in_flight(min(NSTAGE, n_my));
+        const u32x4* st4 = reinterpret_cast<const u32x4*>(my_staging);
         if constexpr (APPEND) {
-            norm_rope_row(qp, a.norm_w, a.sin_cache + (int64_t)(seq_len - 1) * 64, a.cos_cache + (int64_t)(seq_len - 1) * 64,
-                          a.eps, kg, qb);
-        } else {
+            // Four rows at a time, one per DPP row.
 #pragma unroll
-            for (int j = 0; j < 4; ++j) qb[j] = *reinterpret_cast<const u32x4*>(qp + kg * 8 + j * 32);
-        }
+            for (int b4 = 0; b4 < kQSlots; ++b4)
+                norm_rope_rows_lds(my_staging + kQOff, my_staging, my_staging + 512, my_staging + 768, 4 * b4 + kg, n16, a.eps);
+            // Fused append: the last tile of the last split holds the new token. Its K row
+            // (normalised + rotated here) and V row are used from registers and stored to
+            // the cache by the wave that owns that tile.
+            if (holds_new_row) {
+                norm_rope_rows_lds(my_staging + 1024, my_staging + 256, my_staging + 512, my_staging + 768, 0, n16,
+                                   a.eps);  // all four DPP rows work on the one row
 #pragma unroll
-        for (int j = 0; j < 4; ++j) qb[j] = live ? qb[j] : u32x4{0u, 0u, 0u, 0u};
-    }
-    // Fused append: the last tile of the last split holds the new token. Its K row
-    // (normalised + rotated here) and V row are used from registers and stored to
-    // the cache by the wave that owns that tile.
-    if constexpr (APPEND) {
-        if (holds_new_row) {
-            norm_rope_row(a.k_new + kvh * kHeadDim, a.norm_w + kHeadDim, a.sin_cache + (int64_t)(seq_len - 1) * 64,
-                          a.cos_cache + (int64_t)(seq_len - 1) * 64, a.eps, kg, k_fresh);
-            v_fresh = *reinterpret_cast<const u32x4*>(a.v_new + kvh * kHeadDim + n16 * 8);
+                for (int j = 0; j < 4; ++j) k_fresh[j] = st4[64 + j * 4 + kg];
+                v_fresh = st4[64 + 16 + n16];
+            }
+        }
+        const int hq_local = min(n16, a.group - 1);
+        const bool live = n16 < a.group;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u32x4 qv = st4[kQOff / 16 + hq_local * 16 + j * 4 + kg];
+            qb[j] = live ? qv : u32x4{0u, 0u, 0u, 0u};
         }
     }
-
-    // Pin the point where the query (and the fresh rows) must have arrived: here,
-    // before the loop. Left to itself the compiler waits for them at their first use
-    // inside the loop with vmcnt(0) on every trip -- it cannot see the LDS-DMA loads
-    // issued after them -- and that would also wait for every prefetched tile.
-    asm volatile("" ::"v"(qb[0]), "v"(qb[1]), "v"(qb[2]), "v"(qb[3]));
-    if constexpr (APPEND)
-        asm volatile("" ::"v"(k_fresh[0]), "v"(k_fresh[1]), "v"(k_fresh[2]), "v"(k_fresh[3]), "v"(v_fresh));
 
     int stage = 0;
     for (int i = 0; i < n_my; ++i) {
