@@ -321,15 +321,21 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     constexpr int kMergeTail = (2 * NW * G + 2 * G) * (int)sizeof(float);
     constexpr int kCombineBase = kRingBytes + ((kMergeTail + 15) & ~15);
     constexpr int kCombineBytes = (G * kMaxSplits + G + NW) * (int)sizeof(float) + NW * 64 * 16;
-    // Per wave, 1 KiB LDS-DMA slots for the small operands: the query rows of the group (16 chunks
-    // of 16 bytes per head, four heads to a slot) and, in the append variant in front of them, the
-    // operands of the fused QK-Norm + RoPE (slot 0: q_norm | k_norm | sin row | cos row, 16 chunks
-    // each; slot 1: new K row | new V row).
+    // 1 KiB LDS-DMA slots for the small operands. Per wave: the query rows of the group (16 chunks
+    // of 16 bytes per head, four heads to a slot; normalised in place in the append variant).
+    // Append variant, in front of them and shared by the workgroup (every wave fills them with
+    // the same bytes and waits only for its own loads): slot 0 = q_norm | k_norm | sin row |
+    // cos row, 16 chunks each; slot 1 = new K row | new V row, used by one wave only. The slots
+    // lie over the combine area, which nobody touches before the barrier of the epilogue, so they
+    // cost no LDS: with more than 80 KiB per workgroup the compiler assumes one wave per SIMD, puts
+    // the MFMA accumulators into AGPRs and copies all 32 of them to VGPRs and back around the
+    // rescaling of every tile.
     constexpr int kQSlots = (G * 16 + 63) / 64;
-    constexpr int kQOff = APPEND ? 2048 : 0;
-    constexpr int kStageSlots = kQSlots + (APPEND ? 2 : 0);
-    constexpr int kStagingBase = (kCombineBase + kCombineBytes + 1023) & ~1023;
-    constexpr int kSmemBytes = kStagingBase + NW * kStageSlots * 1024;
+    constexpr int kSharedSlots = APPEND ? 2 : 0;
+    constexpr int kStagingBase = (kCombineBase + 1023) & ~1023;
+    constexpr int kStagingBytes = (kSharedSlots + NW * kQSlots) * 1024;
+    constexpr int kSmemBytes =
+        kCombineBase + kCombineBytes > kStagingBase + kStagingBytes ? kCombineBase + kCombineBytes : kStagingBase + kStagingBytes;
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * (NSTAGE * kStageBytes);
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;  // low 32 bits of a flat LDS address = LDS offset
@@ -439,28 +445,30 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     // and the first tile is worked on as soon as it lands. As ordinary loads their wait would be
     // placed by the compiler, which does not know about the DMA loads: it would also wait for
     // every tile issued before that point.
-    char* my_staging = smem + kStagingBase + wave * (kStageSlots * 1024);
+    char* shared_staging = smem + kStagingBase;                                     // append variant only
+    char* my_rows = smem + kStagingBase + (kSharedSlots + wave * kQSlots) * 1024;  // this wave's query rows
     {
-        const uint32_t st = (uint32_t)(uintptr_t)my_staging;
+        const uint32_t st = (uint32_t)(uintptr_t)shared_staging;
+        const uint32_t st_rows = (uint32_t)(uintptr_t)my_rows;
         const int c16 = lane & 15, which = lane >> 4;
         if constexpr (APPEND) {
             const float* sin_row = a.sin_cache + (int64_t)(seq_len - 1) * 64;
             const float* cos_row = a.cos_cache + (int64_t)(seq_len - 1) * 64;
-            const void* p0 = which == 0   ? static_cast<const void*>(a.norm_w + c16 * 8)
-                             : which == 1 ? static_cast<const void*>(a.norm_w + kHeadDim + c16 * 8)
-                             : which == 2 ? static_cast<const void*>(sin_row + c16 * 4)
-                                          : static_cast<const void*>(cos_row + c16 * 4);
-            dma16_gather(p0, st);
+            // (integer selects: as pointer conditionals this becomes a chain of branches)
+            const uint64_t w_base = reinterpret_cast<uint64_t>(a.norm_w) + (uint64_t)(which & 1) * 256u;
+            const uint64_t t_base = reinterpret_cast<uint64_t>(which == 2 ? sin_row : cos_row);
+            const uint64_t p0 = (which < 2 ? w_base : t_base) + (uint64_t)c16 * 16u;
+            dma16_gather(reinterpret_cast<const void*>(p0), st);
             if (holds_new_row) {
-                const void* p1 = (which & 1) == 0 ? static_cast<const void*>(a.k_new + kvh * kHeadDim + c16 * 8)
-                                                  : static_cast<const void*>(a.v_new + kvh * kHeadDim + c16 * 8);
-                dma16_gather(p1, st + 1024);
+                const uint64_t p1 = reinterpret_cast<uint64_t>((which & 1) == 0 ? a.k_new : a.v_new) +
+                                    (uint64_t)(kvh * kHeadDim * 2 + c16 * 16);
+                dma16_gather(reinterpret_cast<const void*>(p1), st + 1024);
             }
         }
 #pragma unroll
         for (int i = 0; i < kQSlots; ++i) {
             const int head = min(which + 4 * i, a.group - 1);  // chunk lane + 64*i: head (lane + 64*i) / 16
-            dma16_gather(a.q + (int64_t)(kvh * a.group + head) * kHeadDim + c16 * 8, st + kQOff + i * 1024);
+            dma16_gather(a.q + (int64_t)(kvh * a.group + head) * kHeadDim + c16 * 8, st_rows + i * 1024);
         }
     }
 #pragma unroll
@@ -471,28 +479,29 @@ __global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) voi
     {
         // Everything issued before the tiles has landed once only the tiles are in flight.
         wait_tiles_in_flight(min(NSTAGE, n_my));
-        const u32x4* st4 = reinterpret_cast<const u32x4*>(my_staging);
+        const u32x4* sh4 = reinterpret_cast<const u32x4*>(shared_staging);
+        const u32x4* rows4 = reinterpret_cast<const u32x4*>(my_rows);
         if constexpr (APPEND) {
             // Four rows at a time, one per DPP row.
 #pragma unroll
             for (int b4 = 0; b4 < kQSlots; ++b4)
-                norm_rope_rows_lds(my_staging + kQOff, my_staging, my_staging + 512, my_staging + 768, 4 * b4 + kg, n16, a.eps);
+                norm_rope_rows_lds(my_rows, shared_staging, shared_staging + 512, shared_staging + 768, 4 * b4 + kg, n16, a.eps);
             // Fused append: the last tile of the last split holds the new token. Its K row
             // (normalised + rotated here) and V row are used from registers and stored to
             // the cache by the wave that owns that tile.
             if (holds_new_row) {
-                norm_rope_rows_lds(my_staging + 1024, my_staging + 256, my_staging + 512, my_staging + 768, 0, n16,
+                norm_rope_rows_lds(shared_staging + 1024, shared_staging + 256, shared_staging + 512, shared_staging + 768, 0, n16,
                                    a.eps);  // all four DPP rows work on the one row
 #pragma unroll
-                for (int j = 0; j < 4; ++j) k_fresh[j] = st4[64 + j * 4 + kg];
-                v_fresh = st4[64 + 16 + n16];
+                for (int j = 0; j < 4; ++j) k_fresh[j] = sh4[64 + j * 4 + kg];
+                v_fresh = sh4[64 + 16 + n16];
             }
         }
         const int hq_local = min(n16, a.group - 1);
         const bool live = n16 < a.group;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const u32x4 qv = st4[kQOff / 16 + hq_local * 16 + j * 4 + kg];
+            const u32x4 qv = rows4[hq_local * 16 + j * 4 + kg];
             qb[j] = live ? qv : u32x4{0u, 0u, 0u, 0u};
         }
     }
