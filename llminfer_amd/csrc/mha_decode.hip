@@ -250,7 +250,7 @@ __device__ __forceinline__ void norm_rope_rows_lds(char* rows, const char* w, co
 }
 
 template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
-__global__ __launch_bounds__(NW * 64, (G >= 16 ? 1 : LLMI_MIN_WAVES_PER_EU)) void mha_decode_kernel(KernelArgs a) {
+__global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
