@@ -96,10 +96,12 @@ static int validate_mha(const llmi_mha_args* a) {
 }
 
 // `wave_cap`: most wavefronts per workgroup the caller's kernel variant supports.
-static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kMaxWaves) {
+// `new_rows`: positions at the end of 0..pos that the kernel takes from registers instead of streaming
+// them from the cache (1 in the append variant): the plan covers the others.
+static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kMaxWaves, int new_rows = 0) {
     if (int rc = validate_mha(a)) return rc;
-    const int seq_len = a->pos + 1;
-    const int tiles = ceil_div(seq_len, kTile);
+    const int seq_len = a->pos + 1 - new_rows;
+    const int tiles = seq_len > 0 ? ceil_div(seq_len, kTile) : 1;  // (nothing cached yet: one workgroup all the same)
     const int n_kv = a->kv_dim / a->head_dim;
     const int group_pad = pow2_ceil(a->kv_mul);
     int max_waves = pow2_floor(kMaxGroupWaves / group_pad);
@@ -207,7 +209,7 @@ int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
     if (!(args->eps >= 0.0f)) return LLMI_ERR_INVALID_ARG;
     if (args->mha.force_path == LLMI_PATH_SPLIT || args->mha.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
     llmi_mha_plan plan;
-    if (int rc = make_plan(&args->mha, &plan, 4)) return rc;
+    if (int rc = make_plan(&args->mha, &plan, 4, 1)) return rc;
     if (plan.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
     return launch_mha_decode(args->mha, plan, args);
 }

@@ -265,25 +265,26 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
     // With a position read from device memory the grid was sized for the largest position:
     // the same rule is applied to the tiles there are, and splits beyond the tile count leave
     // at once.
+    // Append variant: the new token's row never comes from the cache (its K and V are in registers
+    // and go straight into the running softmax of one wave), so the tiles cover positions 0 .. pos-1.
     int seq_len = a.seq_len, n_active = a.num_splits;
     if constexpr (DYN) {
         seq_len = max(0, min(*a.pos_dev, a.seq_len - 1)) + 1;
-        n_active = min(a.num_splits, (seq_len + kTile - 1) / kTile);
+        n_active = min(a.num_splits, max(1, (seq_len - (APPEND ? 1 : 0) + kTile - 1) / kTile));
         if (split >= n_active) return;
     }
-    const int total_tiles = (seq_len + kTile - 1) / kTile;
-    const int run = total_tiles / n_active;     // >= 1: the host never asks for more splits than tiles
+    const int cached_len = seq_len - (APPEND ? 1 : 0);  // positions streamed from the cache
+    const int total_tiles = (cached_len + kTile - 1) / kTile;
+    const int run = total_tiles / n_active;     // the host never asks for more splits than tiles (0 tiles: 1 split)
     const int longer = total_tiles % n_active;  // splits 0 .. longer-1 take run + 1 tiles
     const int ntiles = run + (split < longer ? 1 : 0);
     const int begin = (split * run + min(split, longer)) * kTile;
-    const int nrows = min(ntiles * kTile, seq_len - begin);  // > 0
+    const int nrows = min(ntiles * kTile, cached_len - begin);  // > 0 unless nothing is cached yet
 
     // Filled in below, once the first tiles are on their way.
     u32x4 qb[4];                       // query group, MFMA B operand
-    u32x4 k_fresh[4] = {};             // append variant: the new token's K row (operand layout) ...
-    u32x4 v_fresh = {0u, 0u, 0u, 0u};  // ... and V row chunk
-    // Append variant: the wave that owns the last tile of the last split holds the new token.
-    const bool holds_new_row = APPEND && split == n_active - 1 && ((ntiles - 1) & (NW - 1)) == wave;
+    // Append variant: wave 0 of the last split (the one with the shortest run) takes the new token.
+    const bool holds_new_row = APPEND && split == n_active - 1 && wave == 0;
 
     // Wave-uniform 64-bit bases of this split; lanes add 32-bit byte offsets
     // (scalar-base + vector-offset addressing, no 64-bit multiplies per load).
@@ -486,16 +487,9 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
 #pragma unroll
             for (int b4 = 0; b4 < kQSlots; ++b4)
                 norm_rope_rows_lds(my_rows, shared_staging, shared_staging + 512, shared_staging + 768, 4 * b4 + kg, n16, a.eps);
-            // Fused append: the last tile of the last split holds the new token. Its K row
-            // (normalised + rotated here) and V row are used from registers and stored to
-            // the cache by the wave that owns that tile.
-            if (holds_new_row) {
+            if (holds_new_row)  // the new K row: all four DPP rows work on the one row
                 norm_rope_rows_lds(shared_staging + 1024, shared_staging + 256, shared_staging + 512, shared_staging + 768, 0, n16,
-                                   a.eps);  // all four DPP rows work on the one row
-#pragma unroll
-                for (int j = 0; j < 4; ++j) k_fresh[j] = sh4[64 + j * 4 + kg];
-                v_fresh = sh4[64 + 16 + n16];
-            }
+                                   a.eps);
         }
         const int hq_local = min(n16, a.group - 1);
         const bool live = n16 < a.group;
@@ -504,6 +498,44 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
             const u32x4 qv = rows4[hq_local * 16 + j * 4 + kg];
             qb[j] = live ? qv : u32x4{0u, 0u, 0u, 0u};
         }
+        // Fused append: this wave files the new token's K row (normalised + rotated above) and V
+        // row in the cache and starts its running softmax from that one position -- score q.k,
+        // weight 1, output = the V row -- while its first tiles are still on their way.
+        if constexpr (APPEND) {
+            if (holds_new_row) {
+                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                u32x4 kf[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) kf[j] = sh4[64 + j * 4 + kg];  // operand layout, as a K row of a tile
+                const u32x4 vf = sh4[64 + 16 + n16];                          // columns 8*n16 .. +7
+                if (n16 == 0) {
+                    uint16_t* kd = const_cast<uint16_t*>(a.k) + (int64_t)(seq_len - 1) * a.row_stride + kvh * a.slot_head_stride;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = kf[j];
+                }
+                if (kg == 0)
+                    *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + (int64_t)(seq_len - 1) * a.row_stride +
+                                              kvh * a.slot_head_stride + n16 * 8) = vf;
+                float dot = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const uint32_t qw = qb[j][c], kw = kf[j][c];  // (bit_cast straight from a vector element reads element 0)
+                        dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, qw), __builtin_bit_cast(bf16x2, kw), dot, false);
+                    }
+                dot += __shfl_xor(dot, 16);
+                dot += __shfl_xor(dot, 32);
+                m_run = dot * a.scale_log2e;
+                l_run = kg == 0 ? 1.0f : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t vw = vf[j >> 1];
+                    const float vj = (j & 1) ? bf16_hi(vw) : bf16_lo(vw);
+                    o[j] = f32x4{vj, vj, vj, vj};
+                }
+            }
+        }
     }
 
     int stage = 0;
@@ -511,27 +543,6 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
         TileRegs r;
         wait_tiles_in_flight(min(NSTAGE - 1, n_my - 1 - i));
         read_tile(stage, r);
-        if constexpr (APPEND) {
-            const int t = tile_of(i);
-            if (holds_new_row && t == ntiles - 1) {
-                // Row `fresh` of this tile is the new token; the rows after it are
-                // clamped re-reads of its (still unwritten) cache slot: give them
-                // all the fresh data, the softmax mask drops the extra ones.
-                const int fresh = (nrows - 1) - t * kTile;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) r.k[j] = n16 >= fresh ? k_fresh[j] : r.k[j];
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) r.v[q4] = 4 * kg + q4 >= fresh ? v_fresh : r.v[q4];
-                if (n16 == 0) {
-                    uint16_t* kd = const_cast<uint16_t*>(a.k) + (int64_t)(seq_len - 1) * a.row_stride + kvh * a.slot_head_stride;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = k_fresh[j];
-                }
-                if (kg == 0)
-                    *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + (int64_t)(seq_len - 1) * a.row_stride +
-                                              kvh * a.slot_head_stride + n16 * 8) = v_fresh;
-            }
-        }
         if (i + NSTAGE < n_my) issue_tile(tile_of(i + NSTAGE), stage);
         compute_tile(tile_of(i), r);
         stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
