@@ -12,8 +12,8 @@
 // workgroups of one row per wavefront beat fewer, fatter ones (6144 x 2560: 7.1 vs
 // 7.7 us; 2560 x 4096: 5.6 vs 6.9 us): the matrices are a few microseconds of stream
 // and what counts is how fast the whole chip has loads in flight. Products are formed in fp32 by v_dot2_f32_bf16
-// (two bf16 pairs per instruction, fp32 accumulate), the 64 lanes fold with xor
-// shuffles, lane 0 rounds once and writes.
+// (two bf16 pairs per instruction, fp32 accumulate), the 64 lanes fold with DPP row
+// steps and four scalar reads, lane 0 rounds once and writes.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -45,6 +45,24 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     if (x != x) return 0x7fc0;
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// Sum over the 64 lanes, the result in every lane: four DPP steps inside the 16-lane rows
+// (quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror), then the four row sums are read
+// into scalar registers -- no trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_partner(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row_lane0(float x, int row) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16 * row));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_partner<0xB1>(x);
+    x += dpp_partner<0x4E>(x);
+    x += dpp_partner<0x141>(x);
+    x += dpp_partner<0x140>(x);
+    return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
@@ -97,9 +115,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_kernel(GemvArgs a) {
         for (int r = 0; r < kRows; ++r) acc[r] = dot8(xv, __builtin_nontemporal_load(w4[r] + c), acc[r]);
     }
 #pragma unroll
-    for (int r = 0; r < kRows; ++r)
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) acc[r] += __shfl_xor(acc[r], d);
+    for (int r = 0; r < kRows; ++r) acc[r] = wave_sum(acc[r]);
     if (lane < kRows) {
         float sum = acc[0];
 #pragma unroll
