@@ -110,6 +110,31 @@ __device__ __forceinline__ float wave_sum(float x) {
     return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
+// Folds over lanes l, l^16, l^32, l^48 (the four DPP rows), the result in all of them, with the
+// gfx950 lane swaps: v_permlane32_swap / v_permlane16_swap of a register with itself leave the
+// lower-half (even-row) values in one result and the upper-half (odd-row) values in the other,
+// each in both places. Plain VALU instructions: no trip through the LDS crossbar like a shuffle.
+__device__ __forceinline__ float rows_max(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned h0 = h[0], h1 = h[1];
+    const float y = fmaxf(__builtin_bit_cast(float, h0), __builtin_bit_cast(float, h1));
+    const unsigned v = __builtin_bit_cast(unsigned, y);
+    const auto q = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    const unsigned q0 = q[0], q1 = q[1];
+    return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned h0 = h[0], h1 = h[1];
+    const float y = __builtin_bit_cast(float, h0) + __builtin_bit_cast(float, h1);
+    const unsigned v = __builtin_bit_cast(unsigned, y);
+    const auto q = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    const unsigned q0 = q[0], q1 = q[1];
+    return __builtin_bit_cast(float, q0) + __builtin_bit_cast(float, q1);
+}
+
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 
@@ -378,8 +403,7 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
             s[i] = (row0 + i < nrows) ? c[i] * a.scale_log2e : -INFINITY;
             tmax = fmaxf(tmax, s[i]);
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        tmax = rows_max(tmax);
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = fast_exp2(m_run - m_new);
         float p[4];
@@ -524,8 +548,7 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
                         const uint32_t qw = qb[j][c], kw = kf[j][c];  // (bit_cast straight from a vector element reads element 0)
                         dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, qw), __builtin_bit_cast(bf16x2, kw), dot, false);
                     }
-                dot += __shfl_xor(dot, 16);
-                dot += __shfl_xor(dot, 32);
+                dot = rows_sum(dot);
                 m_run = dot * a.scale_log2e;
                 l_run = kg == 0 ? 1.0f : 0.0f;
 #pragma unroll
@@ -551,8 +574,7 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
     // ---- epilogue: fold the workgroup's waves ----
     // The outputs are already summed over a wave's positions; the denominators are
     // per DPP row (kg) and share the running max of their head, so they add up plainly.
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
+    l_run = rows_sum(l_run);
 
     // This wave's ring is drained (every tile it issued was waited for and read).
     typedef float (*MergeS)[G];
