@@ -124,6 +124,13 @@ __device__ __forceinline__ float rows_max(float x) {
     const unsigned q0 = q[0], q1 = q[1];
     return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
 }
+// x[l] + x[l ^ 32] in both lanes.
+__device__ __forceinline__ float halves_sum(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned h0 = h[0], h1 = h[1];
+    return __builtin_bit_cast(float, h0) + __builtin_bit_cast(float, h1);
+}
 __device__ __forceinline__ float rows_sum(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -761,7 +768,7 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
         // One wavefront per head, all the way: poll, then read the head's partials back and write
         // its 128 outputs, without a workgroup barrier (a wave whose records are in need not wait
         // for the others). Lane = (16-byte column, half of the splits); the two halves are added
-        // with one xor shuffle. The partials of the other workgroups were acknowledged before
+        // with one lane swap. The partials of the other workgroups were acknowledged before
         // their records were written; they are read with device-coherent 16-byte loads, a
         // lane's loads all in flight at once.
         if (wave >= a.group) return;
@@ -796,7 +803,7 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
         if (SA <= 16) gather(std::integral_constant<int, 8>{});
         else gather(std::integral_constant<int, 16>{});
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += __shfl_xor(acc[e], 32);
+        for (int e = 0; e < 4; ++e) acc[e] = halves_sum(acc[e]);
         if (part == 0) {
             // A wait that ran out of patience poisons the output rather than returning a partial sum.
             const float inv = arrived ? 1.0f / den : __builtin_nanf("");
