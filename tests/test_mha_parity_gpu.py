@@ -222,3 +222,14 @@ def test_fused_combine_gives_up_with_nan_instead_of_hanging(oracle, dev, kv_mul,
         assert B.lib().llmi_hip_set_poll_limit(prev) == 0
     assert np.all(np.isnan(got16)) and np.all(np.isnan(got32))
     _check(oracle, dev, case, force_path=B.PATH_SPLIT_FUSED, num_splits=8)
+
+
+@pytest.mark.parametrize("ctx,splits,waves", [(8192, 0, 0), (5000, 7, 4), (1000, 3, 1), (3001, 5, 2)])
+def test_position_major_staggered_walk(oracle, dev, ctx, splits, waves):
+    """Position-major layout, several tiles per wavefront: every split starts its walk at a different
+    tile of its run and wraps round (ragged last tiles included); the result is the oracle's."""
+    case = synth.make_case(23, ctx=ctx, **QWEN3_4B)
+    kw = dict(force_path=B.PATH_SPLIT_FUSED, num_splits=splits, waves_per_group=waves) if splits else {}
+    plan = _check(oracle, dev, case, kv_layout=B.KV_LAYOUT_POS_MAJOR, **kw)
+    tiles = (ctx + 15) // 16
+    assert plan.num_splits > 1 and tiles // plan.num_splits >= 2 * plan.waves_per_group  # two or more tiles per wave
