@@ -9,15 +9,19 @@
 //     in the fp32 workspace; either mha_combine_kernel merges them
 //     (log-sum-exp, a second launch) or the workgroup of the last split does,
 //     inside the same launch (fused combine).
-// Two more template switches: APPEND folds the per-token QK-Norm + RoPE and the
-// K/V cache append of the reference's layer loop into the launch, DYN reads the
-// position from device memory so that one captured launch serves every token.
+// Three more template switches: APPEND folds the per-token QK-Norm + RoPE and the
+// K/V cache append of the reference's layer loop into the launch (the new row
+// enters the softmax from registers), DYN reads the position from device memory
+// so that one captured launch serves every token, STAGGER makes the splits of the
+// position-major layout walk their tiles from different starting points.
 //
 // Differences from the reference design, chosen for CDNA4:
 //   * a workgroup serves ALL query heads of its KV head, so K and V are read
 //     from HBM exactly once (the reference re-reads them once per query head,
 //     mha_kernel.cu:67,104);
-//   * K/V tiles stream through per-wave LDS rings filled by LDS-DMA loads;
+//   * K/V tiles stream through per-wave LDS rings filled by LDS-DMA loads; the
+//     query rows (and the append variant's operands) take the same road, issued
+//     ahead of the tiles, so that every wait is a hand-placed vmcnt;
 //   * q.K^T runs on the matrix cores: one v_mfma_f32_16x16x32_bf16 chain per
 //     tile of 16 positions, K rows as the A operand (lane = row, no transpose
 //     needed because the contraction over head_dim is order-free), the query
