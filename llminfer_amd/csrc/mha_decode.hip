@@ -706,10 +706,9 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
     // e^(m_s - M) into the head's row of s_w and the denominator sum l_s * weight -- all from
     // the polled registers. This workgroup's own (max, sum) comes straight from LDS: its
     // record would be the last one to become visible. Returns false if a record never came.
-    auto poll_head_n = [&](int h, float& den_out, auto slots) -> bool {
+    auto wait_records = [&](int h, auto slots, float* m_reg, float* l_reg) -> bool {
         unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         constexpr int kSlots = decltype(slots)::value;  // splits per lane
-        float m_reg[kSlots], l_reg[kSlots];
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) {
             m_reg[j] = -INFINITY;
@@ -739,7 +738,13 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
             if (__all(ok)) break;
             __builtin_amdgcn_s_sleep(2);
         }
-        const bool arrived = __all(ok);
+        return __all(ok);
+    };
+    // From the polled (max, sum) pairs: M = max m_s, the weights e^(m_s - M) into the head's row
+    // of s_w, the denominator sum l_s * weight; the records are zeroed for the next use.
+    auto make_weights = [&](int h, auto slots, const float* m_reg, const float* l_reg) -> float {
+        unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
+        constexpr int kSlots = decltype(slots)::value;
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) mx = fmaxf(mx, m_reg[j]);
@@ -758,7 +763,13 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
                 }
             }
         }
-        den_out = wave_sum(den);
+        return wave_sum(den);
+    };
+    auto poll_head_n = [&](int h, float& den_out, auto slots) -> bool {
+        constexpr int kSlots = decltype(slots)::value;
+        float m_reg[kSlots], l_reg[kSlots];
+        const bool arrived = wait_records(h, slots, m_reg, l_reg);
+        den_out = make_weights(h, slots, m_reg, l_reg);
         return arrived;
     };
     auto poll_head = [&](int h, float& den_out) -> bool {
@@ -777,48 +788,60 @@ __global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_ker
         // lane's loads all in flight at once.
         if (wave >= a.group) return;
         const int h = wave;
-        float den;
-        const bool arrived = poll_head(h, den);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own weights are in LDS
-        __builtin_amdgcn_wave_barrier();
         const int c4 = lane & 31;
         const int part = lane >> 5;
         const int hq = kvh * a.group + h;
         const uint32_t base = (uint32_t)(((int64_t)hq * S * kHeadDim + c4 * 4) * (int64_t)sizeof(float));
         const float* w = s_w + h * kMaxSplits;
-        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        auto gather = [&](auto batch) {
+        auto load_partial = [&](int sp) {
+            const int spc = min(sp, SA - 1);  // in range; the weight drops the repeat
+            return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, base + (uint32_t)spc * (kHeadDim * 4u), 0, kCoherent));
+        };
+        // The first batch of partials is requested as soon as the records are in and travels
+        // while the weights are worked out (they need the maximum over all records first).
+        auto run = [&](auto slots, auto batch) {
+            constexpr int kSlots = decltype(slots)::value;
             constexpr int kBatch = decltype(batch)::value;
-            for (int s0 = part; s0 < SA; s0 += kBatch * 2) {
-                f32x4 v[kBatch];
-                float wv[kBatch];
+            float m_reg[kSlots], l_reg[kSlots];
+            const bool arrived = wait_records(h, slots, m_reg, l_reg);
+            f32x4 v[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) v[j] = load_partial(part + 2 * j);
+            const float den = make_weights(h, slots, m_reg, l_reg);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own weights are in LDS
+            __builtin_amdgcn_wave_barrier();
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                const int sp = part + 2 * j;
+                acc += v[j] * (sp < SA ? w[sp] : 0.0f);
+            }
+            for (int s0 = part + 2 * kBatch; s0 < SA; s0 += kBatch * 2) {
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) v[j] = load_partial(s0 + 2 * j);
 #pragma unroll
                 for (int j = 0; j < kBatch; ++j) {
-                    const int sp = s0 + j * 2;
-                    const int spc = min(sp, SA - 1);  // in range; the weight below drops the repeat
-                    v[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                         ws_rsrc, base + (uint32_t)spc * (kHeadDim * 4u), 0, kCoherent));
-                    wv[j] = sp < SA ? w[sp] : 0.0f;
+                    const int sp = s0 + 2 * j;
+                    acc += v[j] * (sp < SA ? w[sp] : 0.0f);
                 }
+            }
 #pragma unroll
-                for (int j = 0; j < kBatch; ++j) acc += v[j] * wv[j];
+            for (int e = 0; e < 4; ++e) acc[e] = halves_sum(acc[e]);
+            if (part == 0) {
+                // A wait that ran out of patience poisons the output rather than returning a partial sum.
+                const float inv = arrived ? 1.0f / den : __builtin_nanf("");
+                const f32x4 r = acc * inv;
+                *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
+                if (a.out_f32) {
+                    float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) of[e] = r[e];
+                }
             }
         };
-        if (SA <= 16) gather(std::integral_constant<int, 8>{});
-        else gather(std::integral_constant<int, 16>{});
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] = halves_sum(acc[e]);
-        if (part == 0) {
-            // A wait that ran out of patience poisons the output rather than returning a partial sum.
-            const float inv = arrived ? 1.0f / den : __builtin_nanf("");
-            const f32x4 r = acc * inv;
-            *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
-            if (a.out_f32) {
-                float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
-#pragma unroll
-                for (int e = 0; e < 4; ++e) of[e] = r[e];
-            }
-        }
+        if (SA <= 16) run(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
+        else if (SA <= 64) run(std::integral_constant<int, 1>{}, std::integral_constant<int, 16>{});
+        else run(std::integral_constant<int, kMaxSplits / 64>{}, std::integral_constant<int, 16>{});
         return;
     }
 
