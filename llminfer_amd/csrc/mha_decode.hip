@@ -285,8 +285,15 @@ __device__ __forceinline__ void norm_rope_rows_lds(char* rows, const char* w, co
     *hi_p = u32x2{pack_bf16(oh[0], oh[1]), pack_bf16(oh[2], oh[3])};
 }
 
+// Occupancy hint. Two waves per SIMD keep the register budget at 256, where the compiler picks
+// VGPR-form MFMAs; with the whole file of 512 it keeps the accumulators in AGPRs and copies them to
+// VGPRs and back around the rescaling of every tile. Groups of 16 heads cannot meet the hint in every
+// shape; there it is 1.
+template <int G, int NW>
+constexpr int kWavesPerEu = (G >= 16 && NW != 2) ? 1 : LLMI_MIN_WAVES_PER_EU;
+
 template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
-__global__ __launch_bounds__(NW * 64, LLMI_MIN_WAVES_PER_EU) void mha_decode_kernel(KernelArgs a) {
+__global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kernel(KernelArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
