@@ -221,6 +221,7 @@ struct KernelArgs {
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
     int32_t seq_len;
+    int32_t tiles_run, tiles_longer;  // tiles per split and how many splits take one more (position known on the host)
     int32_t max_polls;             // polls of the fused combine before it gives up and writes NaN
     bool stagger;                  // walk the tiles of a split from a split-dependent starting point (plain variant only)
     int32_t group;        // query heads per KV head
@@ -317,9 +318,14 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
         if (split >= n_active) return;
     }
     const int cached_len = seq_len - (APPEND ? 1 : 0);  // positions streamed from the cache
-    const int total_tiles = (cached_len + kTile - 1) / kTile;
-    const int run = total_tiles / n_active;     // the host never asks for more splits than tiles (0 tiles: 1 split)
-    const int longer = total_tiles % n_active;  // splits 0 .. longer-1 take run + 1 tiles
+    // (the host never asks for more splits than tiles; 0 tiles: 1 split). The division is done on
+    // the host when the position is known there: it is 33 instructions in front of the first load.
+    int run = a.tiles_run, longer = a.tiles_longer;  // splits 0 .. longer-1 take run + 1 tiles
+    if constexpr (DYN) {
+        const int total_tiles = (cached_len + kTile - 1) / kTile;
+        run = total_tiles / n_active;
+        longer = total_tiles % n_active;
+    }
     const int ntiles = run + (split < longer ? 1 : 0);
     const int begin = (split * run + min(split, longer)) * kTile;
     const int nrows = min(ntiles * kTile, cached_len - begin);  // > 0 unless nothing is cached yet
@@ -1050,6 +1056,12 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
     ka.group = args.kv_mul;
     ka.n_q = args.head_num;
     ka.num_splits = plan.num_splits;
+    {
+        const int cached = args.pos + 1 - (append ? 1 : 0);
+        const int tiles = (cached + kTile - 1) / kTile;
+        ka.tiles_run = tiles / plan.num_splits;
+        ka.tiles_longer = tiles % plan.num_splits;
+    }
     ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
     if (append) {
         ka.k_new = static_cast<const uint16_t*>(append->key_new);
