@@ -233,3 +233,20 @@ def test_position_major_staggered_walk(oracle, dev, ctx, splits, waves):
     plan = _check(oracle, dev, case, kv_layout=B.KV_LAYOUT_POS_MAJOR, **kw)
     tiles = (ctx + 15) // 16
     assert plan.num_splits > 1 and tiles // plan.num_splits >= 2 * plan.waves_per_group  # two or more tiles per wave
+
+
+def test_qwen3_32b_head_layout_at_128k(oracle, dev):
+    """64 Q / 8 KV heads at ctx 131072 (512 MiB of K and V, seed 5) at full size against the oracle:
+    the dispatcher's plan (fused combine, one workgroup per CU, 8 waves), the fused combine at the
+    maximum split count, and the two-launch path with the separate combine kernel at 256 splits."""
+    case = synth.make_case(5, n_q=64, n_kv=8, ctx=131072)
+    ref = run_oracle(oracle, case)
+    for kw in (dict(), dict(force_path=B.PATH_SPLIT_FUSED, num_splits=256), dict(force_path=B.PATH_SPLIT, num_splits=256)):
+        got16, got32, plan = run_hip(case, dev, kv_layout=B.KV_LAYOUT_HEAD_MAJOR, want_plan=True, **kw)
+        what = "ctx=131072 path=%d splits=%d waves=%d" % (plan.path, plan.num_splits, plan.waves_per_group)
+        assert_parity(got16, ref, "bf16 out " + what)
+        assert_tap_parity(got32, ref, what)
+        if not kw:
+            assert plan.path == B.PATH_SPLIT_FUSED and plan.num_splits == 32 and plan.waves_per_group == 8
+        else:
+            assert plan.num_splits == 256
