@@ -250,12 +250,15 @@ def _download(ptr, shape, dtype):
     return out
 
 
-@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
-def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout):
-    """4 layers of (QK-Norm + RoPE + append, attention) at ctx 300 + 1 new token: eager run and several
-    replays of the captured graph all match the oracle layer by layer."""
+@pytest.mark.parametrize("layout,layers,ctx", [(B.KV_LAYOUT_POS_MAJOR, 4, 300), (B.KV_LAYOUT_HEAD_MAJOR, 4, 300),
+                                               (B.KV_LAYOUT_HEAD_MAJOR, 36, 4096)])
+def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout, layers, ctx):
+    """Layers of (QK-Norm + RoPE + append, attention) at ctx + 1 new token: eager run and several replays
+    of the captured graph all match the oracle layer by layer. 4 layers at ctx 300 in both layouts, and the
+    Qwen3-4B stack at its full size: 36 layers at ctx 4096 (the caches of the layers are one seeded cache
+    rotated by 37 positions per layer)."""
     H = HostLib()
-    layers, ctx, n_q, n_kv, d = 4, 300, 32, 8, 128
+    n_q, n_kv, d = 32, 8, 128
     msl, pos, kv_dim = ctx + 1, ctx, n_kv * d
     stack = H.L.llmi_host_stack_create(layers, msl, n_q, n_kv, layout)
     assert stack, H.L.llmi_host_last_error().decode()
@@ -265,9 +268,14 @@ def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout):
         k_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
         v_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
         raw = []
+        base = synth.make_case(400, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl) if layers > 4 else None
         for l in range(layers):
-            c = synth.make_case(400 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
-            k_all[l], v_all[l] = c["k"][0], c["v"][0]
+            if base is None:
+                c = synth.make_case(400 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+                k_all[l], v_all[l] = c["k"][0], c["v"][0]
+            else:
+                k_all[l, :ctx] = np.roll(base["k"][0, :ctx], 37 * l, axis=0)
+                v_all[l, :ctx] = np.roll(base["v"][0, :ctx], 37 * l, axis=0)
             qr = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
             kr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
             vr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
