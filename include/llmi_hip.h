@@ -279,6 +279,13 @@ int llmi_hip_abi_version(void);
  * after the call; returns the previous limit. 0 makes every fused launch give up at once: the way to
  * exercise the failure path in a test. */
 int32_t llmi_hip_set_poll_limit(int32_t polls);
+/* No counterpart in the reference. How many of those bounded waits have given up on the current device since
+ * the library was loaded (one count per query head and call; the NaN outputs are the other sign). Reads a
+ * device counter with a synchronous copy: it waits for work already enqueued on the device and must not be
+ * called while a stream is being captured. After a give-up the records that arrived late stay in the
+ * workspace: clear the workspace (llmi_hip_memset_zero) before it is used again by a replay of an
+ * already-captured graph, whose launches carry the same tag; fresh calls get a fresh tag and need nothing. */
+int llmi_hip_poll_timeouts(uint64_t* count);
 const char* llmi_hip_strerror(int status);
 /* The last HIP error string seen by this library on the calling thread ("" if none). */
 const char* llmi_hip_last_error(void);

@@ -4,7 +4,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libllmi_hip.so")
+# LLMI_HIP_LIBRARY names another build of the same library (a tuning or diagnostic variant).
+LIB_PATH = os.environ.get("LLMI_HIP_LIBRARY") or os.path.join(HERE, "libllmi_hip.so")
 
 c_i32 = ctypes.c_int32
 c_void_p = ctypes.c_void_p
@@ -110,6 +111,7 @@ SYMBOLS = {
     "llmi_hip_memset_zero": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, c_i32]),
     "llmi_hip_abi_version": (ctypes.c_int, []),
     "llmi_hip_set_poll_limit": (c_i32, [c_i32]),
+    "llmi_hip_poll_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint64)]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
 }

@@ -53,30 +53,11 @@ def build_host_library(verbose=False):
     return HOST_LIB_PATH
 
 
-def build_host_tests(verbose=False):
-    """tests/host/host_tests: the C++ unit tests of the host layer, linked against both libraries and the oracle."""
-    test_dir = os.path.join(ROOT, "tests", "host")
-    oracle_dir = os.path.join(ROOT, "oracle")
-    subprocess.run(["make", "-C", oracle_dir, "libllmi_oracle.so"], check=True, stdout=subprocess.DEVNULL)
-    hipcc = os.environ.get("HIPCC", "hipcc")
-    exe = os.path.join(test_dir, "host_tests")
-    cmd = [hipcc, "-O1", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument",
-           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(CSRC, "host"), "-I" + oracle_dir,
-           os.path.join(test_dir, "test_host.cpp"),
-           "-L" + HERE, "-lllmi_host", "-lllmi_hip", "-L" + oracle_dir, "-lllmi_oracle",
-           "-Wl,-rpath,$ORIGIN/../../llminfer_amd", "-Wl,-rpath,$ORIGIN/../../oracle", "-o", exe]
-    out = _run(cmd)
-    if verbose and out.strip():
-        print(out)
-    return exe
-
-
 def build_all(verbose=False):
     paths = [build_hip_library(verbose)]
     host = build_host_library(verbose)
     if host:
         paths.append(host)
-        paths.append(build_host_tests(verbose))
     return paths
 
 

@@ -55,15 +55,11 @@ int record_hip_error(hipError_t err, const char* what) {
 }
 
 unsigned long long next_epoch() {
-    // Starts from the clock so that a stale cell left in a reused workspace by
-    // another process run does not match; 48 bits, never 0.
+    // Starts from the clock so that a stale record left in a reused workspace by another process
+    // does not match. record_tag() turns it into a tag that is never zero.
     static std::atomic<unsigned long long> counter{
         (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count()};
-    unsigned long long e;
-    do {
-        e = counter.fetch_add(1, std::memory_order_relaxed) & 0xffffffffffffull;
-    } while (e == 0);
-    return e;
+    return counter.fetch_add(1, std::memory_order_relaxed);
 }
 
 // Default: far beyond any real kernel time (seconds), yet finite.
@@ -367,6 +363,14 @@ int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }
 
 int32_t llmi_hip_set_poll_limit(int32_t polls) {
     return llmi::g_poll_limit.exchange(polls < 0 ? 0 : polls, std::memory_order_relaxed);
+}
+
+int llmi_hip_poll_timeouts(uint64_t* count) {
+    if (!count) return LLMI_ERR_NULL_POINTER;
+    unsigned long long n = 0;
+    if (int rc = read_poll_timeouts(&n)) return rc;
+    *count = n;
+    return LLMI_OK;
 }
 
 const char* llmi_hip_strerror(int status) {

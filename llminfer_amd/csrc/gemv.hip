@@ -19,6 +19,7 @@
 #include <stdint.h>
 
 #include "llmi_internal.h"
+#include "wave_ops.h"
 
 namespace llmi {
 namespace {
@@ -45,24 +46,6 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     if (x != x) return 0x7fc0;
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-}
-
-// Sum over the 64 lanes, the result in every lane: four DPP steps inside the 16-lane rows
-// (quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror), then the four row sums are read
-// into scalar registers -- no trips through the LDS crossbar.
-template <int CTRL>
-__device__ __forceinline__ float dpp_partner(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float row_lane0(float x, int row) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16 * row));
-}
-__device__ __forceinline__ float wave_sum(float x) {
-    x += dpp_partner<0xB1>(x);
-    x += dpp_partner<0x4E>(x);
-    x += dpp_partner<0x141>(x);
-    x += dpp_partner<0x140>(x);
-    return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {

@@ -47,6 +47,8 @@ base::Status WeightFile::open(const std::string& path, std::unique_ptr<WeightFil
     f->payload_ = reinterpret_cast<const uint16_t*>(static_cast<const char*>(map) + header_bytes);  // :177
     f->payload_elems_ = (file_size - header_bytes) / sizeof(uint16_t);
 
+    // (|INT32_MIN| does not exist: a header that says so is not a model)
+    if (f->config_.vocab_size == INT32_MIN) return parse_error("The vocabulary size in the model file is out of range.");
     if (header_ints == 7) {  // header and raw payload only: that file predates the layout below
         f->vocab_size_ = std::abs(f->config_.vocab_size);
         *out = std::move(f);
@@ -59,7 +61,11 @@ base::Status WeightFile::open(const std::string& path, std::unique_ptr<WeightFil
         return parse_error("The configuration in the model file is not positive.");
     if (c.dim % c.head_num != 0) return parse_error("dim is not a multiple of head_num.");            // :221
     f->head_dim_ = c.dim / c.head_num;                                                                  // :222
-    f->kv_dim_ = f->head_dim_ * c.kv_head_num;                                                          // :223
+    // The header is untrusted input: every product below is formed in 64 bits and checked.
+    const int64_t kv_dim64 = static_cast<int64_t>(f->head_dim_) * c.kv_head_num;                       // :223
+    if (kv_dim64 > INT32_MAX || static_cast<int64_t>(c.dim) + 2 * kv_dim64 > INT32_MAX)
+        return parse_error("kv_dim in the model file is out of range.");
+    f->kv_dim_ = static_cast<int32_t>(kv_dim64);
     if (f->head_dim_ % 2 != 0) return parse_error("head_dim is odd.");                                 // :224
     if (c.head_num % c.kv_head_num != 0) return parse_error("head_num is not a multiple of kv_head_num.");  // :226
     f->vocab_size_ = std::abs(c.vocab_size);                                                            // :233
@@ -68,17 +74,31 @@ base::Status WeightFile::open(const std::string& path, std::unique_ptr<WeightFil
     const size_t L = static_cast<size_t>(c.layer_num), hid = static_cast<size_t>(c.hidden_dim);
     const size_t dim = static_cast<size_t>(c.dim), kv = static_cast<size_t>(f->kv_dim_);
     const size_t imm = static_cast<size_t>(c.immediate_dim), hd = static_cast<size_t>(f->head_dim_);
+    // Every tensor has to fit the payload, so a term beyond it (or a product that wraps) ends the walk:
+    // a crafted header cannot make the sum wrap round to the file size.
     size_t off = 0;
-    f->off_embedding_ = off;  off += static_cast<size_t>(f->vocab_size_) * hid;  // 1. embedding
-    f->off_pre_norm_ = off;   off += L * hid;                                    // 2. pre-attention RMSNorm
-    f->off_qkv_ = off;        off += L * (dim + 2 * kv) * hid;                   // 3. packed QKV projection
-    f->off_qk_norm_ = off;    off += L * 2 * hd;                                 // 4. q_norm, k_norm
-    f->off_o_ = off;          off += L * hid * dim;                              // 5. output projection
-    f->off_ffn_norm_ = off;   off += L * hid;                                    // 6. FFN RMSNorm
-    f->off_gate_up_ = off;    off += L * 2 * imm * hid;                          // 7. gate and up projections
-    f->off_down_ = off;       off += L * hid * imm;                              // 8. down projection
-    f->off_final_norm_ = off; off += hid;                                        // 9. final RMSNorm
-    f->total_elems_ = off;                                                       // 10. lm_head is the embedding
+    bool fits = true;
+    const size_t limit = f->payload_elems_;
+    auto advance = [&](size_t a, size_t b, size_t c3) {
+        size_t ab = 0, abc = 0;
+        if (__builtin_mul_overflow(a, b, &ab) || __builtin_mul_overflow(ab, c3, &abc) || abc > limit || off > limit - abc) {
+            fits = false;
+            return;
+        }
+        off += abc;
+    };
+    f->off_embedding_ = off;  advance(static_cast<size_t>(f->vocab_size_), hid, 1);  // 1. embedding
+    f->off_pre_norm_ = off;   advance(L, hid, 1);                                    // 2. pre-attention RMSNorm
+    f->off_qkv_ = off;        advance(L, dim + 2 * kv, hid);                         // 3. packed QKV projection
+    f->off_qk_norm_ = off;    advance(L, 2, hd);                                     // 4. q_norm, k_norm
+    f->off_o_ = off;          advance(L, hid, dim);                                  // 5. output projection
+    f->off_ffn_norm_ = off;   advance(L, hid, 1);                                    // 6. FFN RMSNorm
+    f->off_gate_up_ = off;    advance(L, 2 * imm, hid);                              // 7. gate and up projections
+    f->off_down_ = off;       advance(L, hid, imm);                                  // 8. down projection
+    f->off_final_norm_ = off; advance(hid, 1, 1);                                    // 9. final RMSNorm
+    f->total_elems_ = off;                                                           // 10. lm_head is the embedding
+    if (!fits)
+        return parse_error("The model file is " + std::to_string(file_size) + " bytes, shorter than the tensors its header describes.");
     if (header_bytes + off * sizeof(uint16_t) != file_size)  // :317-318
         return parse_error("The model file is " + std::to_string(file_size) + " bytes, its header describes " +
                            std::to_string(header_bytes + off * sizeof(uint16_t)) + ".");

@@ -48,7 +48,10 @@ public:
     size_t payload_elements() const { return payload_elems_; }
 
     // Start of the payload; element offset `offset` (RawModelDataBf16::weight_ptr).
-    const uint16_t* weight_ptr(size_t offset) const { return payload_ + offset; }
+    const uint16_t* weight_ptr(size_t offset) const {
+        LLMI_CHECK(offset <= payload_elems_);
+        return payload_ + offset;
+    }
     const void* payload_bytes() const { return payload_; }
 
     // The tensors in file order (qwen3_fused.cpp:246-314).

@@ -18,8 +18,14 @@ int record_hip_error(hipError_t err, const char* what);
 // hipGetLastError() after a kernel launch.
 int check_launch();
 
-// A fresh 48-bit tag per decode call (never 0), for the arrival cells of the fused combine.
+// A fresh number per decode call, for the arrival records of the fused combine.
 unsigned long long next_epoch();
+// The 32-bit tag a call's records carry, from its epoch: bit 31 is always set, so that a tag never
+// equals a cleared record (all zero) whatever the epoch counter reads -- also when its low bits wrap
+// to zero; the low 31 bits are the epoch's.
+constexpr uint32_t record_tag(unsigned long long epoch) { return 0x80000000u | (uint32_t)(epoch & 0x7fffffffull); }
+// Waits of the fused combine that gave up since the library was loaded (device counter of the current device).
+int read_poll_timeouts(unsigned long long* count);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.
 int poll_limit();
 

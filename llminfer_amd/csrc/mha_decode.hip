@@ -50,6 +50,7 @@
 #include <type_traits>
 
 #include "llmi_internal.h"
+#include "wave_ops.h"
 
 namespace llmi {
 
@@ -61,8 +62,14 @@ typedef short i16x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
+// Waits of the fused combine that ran out of polls, counted on the device (one per head and call).
+__device__ unsigned int g_poll_timeouts = 0;
+
 constexpr int kTile = 16;      // positions per MFMA tile
 constexpr int kHeadDim = 128;
+// Cache policy of the buffer loads and stores that hand partial results from one workgroup to
+// another: the instruction's sc1 bit, device scope (served by memory, coherent across the XCDs).
+constexpr int kCacheDevice = 16;
 // Build-time tuning knobs.
 #ifndef LLMI_NT_LOADS
 #define LLMI_NT_LOADS 1  // K/V are read once: stream them past the caches
@@ -85,33 +92,6 @@ template <int SRC>
 __device__ __forceinline__ float row_bcast(float x) {
     return __builtin_bit_cast(
         float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + SRC, 0xf, 0xf, false));
-}
-
-// x of the lane's DPP partner: quad_perm [1,0,3,2] (0xB1), [2,3,0,1] (0x4E), row_half_mirror (0x141),
-// row_mirror (0x140). Applied in this order with a commutative fold they leave the fold of all 16
-// lanes of a row in every lane, at VALU speed.
-template <int CTRL>
-__device__ __forceinline__ float dpp_partner(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float row_lane0(float x, int row) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16 * row));
-}
-// Folds over all 64 lanes, the result in every lane: four DPP steps inside the rows, then the four
-// row results are read into scalar registers (no LDS-crossbar shuffles, whose latency adds up).
-__device__ __forceinline__ float wave_max(float x) {
-    x = fmaxf(x, dpp_partner<0xB1>(x));
-    x = fmaxf(x, dpp_partner<0x4E>(x));
-    x = fmaxf(x, dpp_partner<0x141>(x));
-    x = fmaxf(x, dpp_partner<0x140>(x));
-    return fmaxf(fmaxf(row_lane0(x, 0), row_lane0(x, 1)), fmaxf(row_lane0(x, 2), row_lane0(x, 3)));
-}
-__device__ __forceinline__ float wave_sum(float x) {
-    x += dpp_partner<0xB1>(x);
-    x += dpp_partner<0x4E>(x);
-    x += dpp_partner<0x141>(x);
-    x += dpp_partner<0x140>(x);
-    return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
 // Folds over lanes l, l^16, l^32, l^48 (the four DPP rows), the result in all of them, with the
@@ -172,6 +152,8 @@ __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t 
     // The instruction takes its base and the LDS offset (through M0) from scalar
     // registers; readfirstlane guarantees that whatever the surrounding code
     // made of these wave-uniform values (it is free when they already are scalar).
+    // M0 is an operand of the asm statement (constraint {m0}): the compiler writes it and
+    // knows that it is live; the s_nop covers the wait state between that write and the load.
     const uint64_t b = reinterpret_cast<uint64_t>(base);
     // (the builtin returns a signed int: go through uint32_t so that the low half is not sign-extended)
     const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
@@ -179,11 +161,9 @@ __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t 
     const uint64_t sbase = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
     const uint32_t slds = (uint32_t)__builtin_amdgcn_readfirstlane(lds_off);
 #if LLMI_NT_LOADS
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
-                 :: "s"(slds), "v"(voff), "s"(sbase) : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" :: "v"(voff), "s"(sbase), "{m0}"(slds) : "memory");
 #else
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(slds), "v"(voff), "s"(sbase) : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "{m0}"(slds) : "memory");
 #endif
 }
 
@@ -191,8 +171,7 @@ __device__ __forceinline__ void dma16(const char* base, uint32_t voff, uint32_t 
 // operands that many workgroups share (they stay in L2).
 __device__ __forceinline__ void dma16_gather(const void* ptr, uint32_t lds_off) {
     const uint32_t slds = (uint32_t)__builtin_amdgcn_readfirstlane(lds_off);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :: "s"(slds), "v"(ptr) : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(ptr), "{m0}"(slds) : "memory");
 }
 
 // Waits until at most `newer_tiles` whole tiles (8 loads each) are still in flight.
@@ -216,7 +195,7 @@ struct KernelArgs {
     uint16_t* out;        // [n_kv*group][128]
     float* out_f32;       // optional
     unsigned long long* records;   // [n_q][num_splits][2] arrival records of the fused combine, or nullptr
-    unsigned long long epoch;      // tag of this call, 48 bits
+    uint32_t tag;                  // record tag of this call: see record_tag()
     const int32_t* pos_dev;        // optional: position read at run time (seq_len then is its upper bound + 1)
     int32_t row_stride;   // elements between consecutive positions of one KV head
     int64_t head_stride;  // elements between KV heads
@@ -299,8 +278,13 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
     const int kg = lane >> 4;   // MFMA k-group / DPP row
-    const int split = blockIdx.x;
-    const int kvh = blockIdx.y;
+    // Workgroups are handed to the eight XCDs (each with its own L2) in turn, in index order with x
+    // fastest: with the KV head in x, the splits of a head land on one XCD whenever the number of
+    // KV heads is a multiple of eight, and the combiners (last splits) spread over all of them
+    // instead of sharing one. Nothing relies on that placement for correctness; it is worth
+    // 0.1-0.35 us per call (32 query / 8 KV heads, 1K to 32K positions) against split-fastest.
+    const int kvh = blockIdx.x;
+    const int split = blockIdx.y;
 
     // A KV head's 16-position tiles are dealt to the splits in contiguous runs whose lengths
     // differ by at most one tile (the first tiles % S splits get the longer run), so every split
@@ -671,7 +655,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     if (c4 == 0) {
                         unsigned long long* rec = a.records + ((int64_t)hq * S + split) * 2;
-                        const unsigned long long tag = a.epoch & 0xffffffffull;
+                        const unsigned long long tag = a.tag;
                         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, mx);
                         const unsigned long long l_bits = __builtin_bit_cast(uint32_t, lsum);
                         __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -706,7 +690,6 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     // graph replay of this very call (same epoch) starts clean.
     const int S = a.num_splits;  // layout stride of partials and records
     const int SA = n_active;     // splits that hold positions
-    const unsigned long long tag = a.epoch & 0xffffffffull;
     if (split != SA - 1) return;  // (its records went out above)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the combiner's own partial stores are acknowledged
     __syncthreads();                                  // ... and its (max, sum) pairs are in LDS
@@ -715,12 +698,11 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     float* s_den = s_w + G * kMaxSplits;                         // [G] denominators
     int* s_ok = reinterpret_cast<int*>(s_den + G);               // [NW] every record seen
     f32x4* s_part = reinterpret_cast<f32x4*>(s_ok + NW);         // [NW * 64] per-thread partial sums
-    // Waits for the records of head h (one wavefront does), then M = max m_s, weights
-    // e^(m_s - M) into the head's row of s_w and the denominator sum l_s * weight -- all from
-    // the polled registers. This workgroup's own (max, sum) comes straight from LDS: its
-    // record would be the last one to become visible. Returns false if a record never came.
+    // Waits for the records of head h (one wavefront does); the (max, sum) pairs stay in the polling
+    // lanes' registers. This workgroup's own pair comes straight from LDS: its record would be the
+    // last one to become visible. Returns false if a record never came. A record only counts when
+    // it carries this call's tag (never zero, which is what a cleared record holds).
     auto wait_records = [&](int h, auto slots, float* m_reg, float* l_reg) -> bool {
-        unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         constexpr int kSlots = decltype(slots)::value;  // splits per lane
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) {
@@ -730,6 +712,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
         bool ok = false;
         // Bounded wait: every wave leaves this loop even if a record never shows up
         // (the result is then poisoned below instead of hanging the GPU).
+        unsigned long long* rec = a.records + (int64_t)(kvh * a.group + h) * S * 2;
         for (int spin = 0; spin < a.max_polls; ++spin) {
             ok = true;
 #pragma unroll
@@ -740,7 +723,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
                 if (sp < SA - 1) {
                     const unsigned long long r0 = __hip_atomic_load(rec + 2 * sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     const unsigned long long r1 = __hip_atomic_load(rec + 2 * sp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ok = ok && (r0 & 0xffffffffull) == tag && (r1 & 0xffffffffull) == tag;
+                    ok = ok && (uint32_t)r0 == a.tag && (uint32_t)r1 == a.tag;
                     m_reg[j] = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
                     l_reg[j] = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
                 } else if (sp == SA - 1) {
@@ -751,7 +734,10 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
             if (__all(ok)) break;
             __builtin_amdgcn_s_sleep(2);
         }
-        return __all(ok);
+        const bool arrived = __all(ok);
+        // A give-up is counted where the host can read it (llmi_hip_poll_timeouts).
+        if (!arrived && lane == 0) atomicAdd(&g_poll_timeouts, 1u);
+        return arrived;
     };
     // From the polled (max, sum) pairs: M = max m_s, the weights e^(m_s - M) into the head's row
     // of s_w, the denominator sum l_s * weight; the records are zeroed for the next use.
@@ -790,7 +776,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
         return poll_head_n(h, den_out, std::integral_constant<int, kMaxSplits / 64>{});
     };
     const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
-    constexpr int kCoherent = 16;  // cache policy: sc1
+    constexpr int kCoherent = kCacheDevice;
 
     if (a.group <= NW) {
         // One wavefront per head, all the way: poll, then read the head's partials back and write
@@ -952,8 +938,7 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
 
     float mx = -INFINITY;
     for (int s = tid; s < num_splits; s += kHeadDim) mx = fmaxf(mx, ms[s]);
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    mx = wave_max(mx);
     if ((tid & 63) == 0) s_red[tid >> 6] = mx;
     __syncthreads();
     mx = fmaxf(s_red[0], s_red[1]);
@@ -966,8 +951,7 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
         s_w[s] = f;
         lsum += ls[s] * f;
     }
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) lsum += __shfl_xor(lsum, d);
+    lsum = wave_sum(lsum);
     if ((tid & 63) == 0) s_red[tid >> 6] = lsum;
     __syncthreads();
     lsum = s_red[0] + s_red[1];
@@ -991,7 +975,7 @@ template <int G, int NW>
 void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stream) {
     // NW * NSTAGE * 8 KiB of ring must fit the LDS budget of one workgroup.
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
-    dim3 grid(ka.num_splits, n_kv);
+        dim3 grid(n_kv, ka.num_splits);
     const bool dyn = ka.pos_dev != nullptr;  // position read at run time: its own instantiation, the static one pays nothing
     if (append) {
         if constexpr (NW <= 4) {
@@ -1022,6 +1006,14 @@ bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipSt
 
 }  // namespace
 
+int read_poll_timeouts(unsigned long long* count) {
+    unsigned int n = 0;
+    if (int rc = record_hip_error(hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_poll_timeouts), sizeof(n)), "hipMemcpyFromSymbol"))
+        return rc;
+    *count = n;
+    return LLMI_OK;
+}
+
 int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append) {
     const int n_kv = args.kv_dim / args.head_dim;
     const int64_t layer_off = (int64_t)args.layer_id * args.max_seq_len * args.kv_dim;
@@ -1034,14 +1026,14 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
     ka.out = static_cast<uint16_t*>(args.output);
     ka.out_f32 = args.output_f32;
     ka.records = nullptr;
-    ka.epoch = 0;
+    ka.tag = 0;
     ka.pos_dev = args.pos_device;
     if (plan.path == LLMI_PATH_SPLIT_FUSED) {
         // Arrival records sit behind the partial outputs in the workspace.
         const size_t partial_bytes = (size_t)args.head_num * plan.num_splits * args.head_dim * sizeof(float);
         ka.records = reinterpret_cast<unsigned long long*>(static_cast<char*>(args.workspace) +
                                                            ((partial_bytes + 15) & ~(size_t)15));
-        ka.epoch = next_epoch();
+        ka.tag = record_tag(next_epoch());
     }
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
         ka.row_stride = args.kv_dim;

@@ -7,12 +7,13 @@
 //   * the sin/cos table (role of sin_cos_cache_kernel, code/source/op/kernel/cuda/rope_kernel.cu:6-21);
 //   * a position-major -> head-major cache copy.
 // One wavefront per head: lane i owns the rotation pair (i, i+64), the sum of
-// squares is reduced across the 64 lanes with xor shuffles, no LDS.
+// squares is folded across the 64 lanes with DPP row steps and scalar reads, no LDS.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include "llmi_internal.h"
+#include "wave_ops.h"
 
 namespace llmi {
 namespace {
@@ -73,8 +74,7 @@ __global__ __launch_bounds__(kHalf) void qk_norm_rope_append_kernel(AppendArgs a
     const float x0 = bf16_to_f32(src[i]);
     const float x1 = bf16_to_f32(src[i + kHalf]);
     float ss = x0 * x0 + x1 * x1;
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) ss += __shfl_xor(ss, d);
+    ss = wave_sum(ss);
     const float r = 1.0f / sqrtf(ss / (float)kHeadDim + a.eps);
     const float av = x0 * bf16_to_f32(w[i]) * r;
     const float bv = x1 * bf16_to_f32(w[i + kHalf]) * r;

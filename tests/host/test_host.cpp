@@ -7,6 +7,7 @@
 //   host_tests gpu   tests that need one
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <random>
@@ -17,6 +18,7 @@
 #include "decode_stack.h"
 #include "kernel_interface.h"
 #include "llmi_hip.h"
+#include "llmi_internal.h"
 #include "llmi_oracle.h"
 #include "mha.h"
 #include "qk_norm_rope.h"
@@ -481,6 +483,57 @@ TEST(gpu_gemv_family_through_the_registry) {
     // operand checks of the shims: wrong output type, wrong inner dimension
     tensor::Tensor bad_out(DataType::DataTypeFp32, hidden, true, hip_alloc());
     EXPECT(is_fatal([&] { kernel::get_fused_gemv_add_kernel(DeviceType::DeviceHIP)(q_d, wo_d, bad_out, cfg->stream); }));
+}
+
+TEST(cpu_pool_policy_over_a_host_backing_allocator) {
+    // The pooled allocator of the C ABI over malloc / free: the reference's two block classes, best fit,
+    // nothing handed back before trim (alloc_cu.cpp:7-119). Under the sanitizer build this walks pool.cpp.
+    struct Counts { int allocs = 0, frees = 0; } counts;
+    auto alloc_fn = [](void** p, size_t n, void* u) -> int { ++static_cast<Counts*>(u)->allocs; *p = std::malloc(n); return *p ? 0 : -1; };
+    auto free_fn = [](void* p, void* u) -> int { ++static_cast<Counts*>(u)->frees; std::free(p); return 0; };
+    llmi_pool* pool = llmi_pool_create(alloc_fn, free_fn, &counts);
+    EXPECT(pool != nullptr);
+    EXPECT(llmi_pool_alloc(pool, 0) == nullptr);
+    void* small1 = llmi_pool_alloc(pool, 1000);
+    void* small2 = llmi_pool_alloc(pool, 5000);
+    void* big1 = llmi_pool_alloc(pool, (3u << 20) + 17);
+    EXPECT(small1 && small2 && big1 && counts.allocs == 3);
+    std::memset(small1, 1, 1000); std::memset(small2, 2, 5000); std::memset(big1, 3, (3u << 20) + 17);
+    EXPECT(llmi_pool_free(pool, small2) == LLMI_OK && llmi_pool_free(pool, big1) == LLMI_OK);
+    EXPECT(llmi_pool_free(pool, small2) == LLMI_ERR_UNKNOWN_POINTER);  // not busy any more
+    int on_stack = 0;
+    EXPECT(llmi_pool_free(pool, &on_stack) == LLMI_ERR_UNKNOWN_POINTER);
+    EXPECT(llmi_pool_free(pool, nullptr) == LLMI_OK);
+    EXPECT(llmi_pool_alloc(pool, 4000) == small2);            // smallest free small block that fits
+    EXPECT(llmi_pool_alloc(pool, 3u << 20) == big1);          // big block reused: slack under 1 MiB
+    void* big2 = llmi_pool_alloc(pool, 1u << 21);
+    EXPECT(big2 && big2 != big1 && counts.allocs == 4);
+    llmi_pool_stats st;
+    EXPECT(llmi_pool_get_stats(pool, &st) == LLMI_OK);
+    EXPECT(st.backing_allocs == 4 && st.reuses == 2 && st.big_busy_blocks == 2 && st.small_busy_blocks == 2);
+    EXPECT(llmi_pool_free(pool, big2) == LLMI_OK);
+    EXPECT(llmi_pool_trim(pool) == (1u << 21) && counts.frees == 1);
+    llmi_pool_destroy(pool);  // hands back what is left, busy or free
+    EXPECT(counts.frees == counts.allocs);
+}
+
+TEST(cpu_record_tag_is_never_zero) {
+    // The tag of a call's arrival records must differ from a cleared record (all zero) for every value of
+    // the 64-bit epoch counter, in particular when its low 32 (or 31) bits wrap to zero.
+    const unsigned long long edges[] = {0ull, 1ull, 0x7fffffffull, 0x80000000ull, 0xffffffffull, 0x100000000ull,
+                                        0x7fffffff00000000ull, 0xffffffff00000000ull, 0xffffffffffffffffull};
+    for (unsigned long long e : edges)
+        for (long long d = -3; d <= 3; ++d) {
+            const unsigned long long epoch = e + (unsigned long long)d;
+            EXPECT(llmi::record_tag(epoch) != 0u);
+            EXPECT((llmi::record_tag(epoch) & 0x80000000u) != 0u);
+            EXPECT(llmi::record_tag(epoch) != llmi::record_tag(epoch + 1));  // consecutive calls never share a tag
+        }
+    // a walk across the 2^32 boundary of the counter
+    for (unsigned long long epoch = 0xfffffff0ull; epoch < 0x100000010ull; ++epoch) EXPECT(llmi::record_tag(epoch) != 0u);
+    // the library's own counter hands out distinct epochs
+    const unsigned long long e0 = llmi::next_epoch(), e1 = llmi::next_epoch();
+    EXPECT(e1 == e0 + 1);
 }
 
 int main(int argc, char** argv) {

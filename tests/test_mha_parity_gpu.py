@@ -1,6 +1,8 @@
 """GPU parity of llmi_hip_mha_decode (through the C ABI) against the CPU oracle
 on the same seeded, bf16-rounded inputs. Gate: |d| <= 2e-3 + 1e-2*|ref| on the
 bf16 output, and max-abs <= 2e-3; the fp32 tap is held to a tighter bound."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -214,6 +216,13 @@ def test_fused_combine_gives_up_with_nan_instead_of_hanging(oracle, dev, kv_mul,
     on the same data gives the oracle's answer. Both merge variants (one wavefront per head, and
     heads shared out when a group has more heads than the workgroup has wavefronts)."""
     case = synth.make_case(31, ctx=1000, n_q=kv_mul * n_kv, n_kv=n_kv)
+
+    def timeouts():
+        n = ctypes.c_uint64()
+        assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(n)) == 0
+        return n.value
+
+    before = timeouts()
     prev = B.lib().llmi_hip_set_poll_limit(0)
     try:
         assert prev == 1 << 22
@@ -221,7 +230,10 @@ def test_fused_combine_gives_up_with_nan_instead_of_hanging(oracle, dev, kv_mul,
     finally:
         assert B.lib().llmi_hip_set_poll_limit(prev) == 0
     assert np.all(np.isnan(got16)) and np.all(np.isnan(got32))
+    # every give-up is counted on the device, one per query head, where the host can read it
+    assert timeouts() == before + kv_mul * n_kv
     _check(oracle, dev, case, force_path=B.PATH_SPLIT_FUSED, num_splits=8)
+    assert timeouts() == before + kv_mul * n_kv  # a call that completes counts nothing
 
 
 @pytest.mark.parametrize("ctx,splits,waves", [(8192, 0, 0), (5000, 7, 4), (1000, 3, 1), (3001, 5, 2)])

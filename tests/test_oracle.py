@@ -2,6 +2,8 @@
 independent float64 evaluation, library routines (torch SDPA, torch bf16 conversion, scipy softmax),
 closed forms, invariants and long-double brute force. Each check is chosen so that a plausible slip
 (dropped scale, wrong KV-head index, transposed operand, off-by-one in pos, wrong rotation sign) fails it."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -325,3 +327,12 @@ def test_gemv_matches_torch_bf16_matmul_rounding(oracle):
     ref = (torch.from_numpy(synth.bf16_bits_to_f32(w)) @ torch.from_numpy(synth.bf16_bits_to_f32(x))).numpy()
     got = oracle.gemv_bf16(x, w)
     assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(synth.bf16_bits_to_f32(w)) @ np.abs(synth.bf16_bits_to_f32(x)))
+
+
+def test_oracle_under_sanitizers():
+    """`make -C oracle asan`: every oracle function over exact-size heap buffers with AddressSanitizer + UBSan."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run(["make", "-C", os.path.join(root, "oracle"), "asan"], stdout=subprocess.PIPE,
+                         stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert res.returncode == 0 and "oracle asan check: ok" in res.stdout, res.stdout[-3000:]

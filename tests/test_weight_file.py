@@ -102,6 +102,25 @@ def test_bad_paths_and_headers(tmp_path):
     assert info(L, q)[0] == 3                                      # dim % head_num != 0 (:221)
 
 
+@pytest.mark.parametrize("cfg", [
+    (256, 64, 2, 2, 1, -2**31, 32, 96),                     # |vocab_size| does not exist
+    (2**30, 2**30, 2**30, 2, 1, 2**30, 32, 2**30),          # every product wraps 64 bits
+    (2**16, 2**31 - 1, 2**31 - 1, 1, 1, 2**31 - 1, 32, 2**31 - 1),
+    (2**31 - 2, 64, 1, 2, 2**31 - 1, 8, 32, 96),            # head_dim * kv_head_num beyond int32
+    (256, 64, 2**31 - 1, 2, 1, 8, 32, 96),                  # plausible shapes, absurd layer count
+])
+def test_overflowing_headers_are_parse_errors(tmp_path, cfg):
+    """The header is untrusted: sizes that wrap 32- or 64-bit arithmetic must not pass the length check
+    (they could make the summed offsets wrap round to the real file size), whatever payload follows."""
+    L = host_lib()
+    p = str(tmp_path / "evil.bin")
+    with open(p, "wb") as f:
+        f.write(np.asarray(cfg, dtype=np.int64).astype(np.int32).tobytes())
+        f.write(b"\0" * 4096)
+    rc, _, _ = info(L, p)
+    assert rc == 3, L.llmi_host_last_error().decode()
+
+
 def test_engine_fixture_with_the_older_header():
     """The engine's own loader fixture (7 x int32 header, then float(i) for i < dim * hidden_dim): the values its
     test expects (test/test_op/test_load.cpp:19-26,52-56)."""
