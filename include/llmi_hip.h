@@ -123,6 +123,22 @@ int llmi_hip_mha_plan(const llmi_mha_args* args, llmi_mha_plan* plan);
  * share a workspace must not overlap in time. */
 int llmi_hip_mha_decode(const llmi_mha_args* args);
 
+/* No counterpart in the reference. For callers that cannot allocate device memory and have no workspace to
+ * pass -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc: the same
+ * computation as llmi_hip_mha_decode with the same results, but the split path's partial results and arrival
+ * records go to a fixed 4 MiB array in device memory that is part of the library's code object (each GPU
+ * the library runs on holds one from its first use until the process ends). `workspace` and
+ * `workspace_bytes` of `args` are ignored. Calls no hipMalloc / hipFree or any other allocating routine.
+ * The array bounds the split count: the automatic plan takes as many splits as fit (what
+ * llmi_hip_mha_decode does with a workspace of that size: head_num * splits * 528 + 16 bytes), a forced
+ * `num_splits` that needs more, or a head count so large that two splits do not fit, is rejected with
+ * LLMI_ERR_WORKSPACE and llmi_hip_last_error() says so. Every call on a GPU shares that GPU's array: two
+ * calls that overlap in time on one GPU (two streams, two threads) race, like two calls of
+ * llmi_hip_mha_decode on one workspace. The array needs no clearing between calls (records carry a per-call
+ * tag). The first call on a device looks the array's address up (which may load the code object): make it
+ * outside stream capture. */
+int llmi_hip_mha_decode_static(const llmi_mha_args* args);
+
 typedef struct llmi_mha_append_args {
     llmi_mha_args mha;        /* as for llmi_hip_mha_decode, except: mha.query is the RAW query of the new
                                  token (before QK-Norm), and the caches are written at (layer_id, pos)  */

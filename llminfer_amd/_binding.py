@@ -91,6 +91,7 @@ BACKING_FREE_FN = ctypes.CFUNCTYPE(ctypes.c_int, c_void_p, c_void_p)
 SYMBOLS = {
     "llmi_hip_mha_plan": (ctypes.c_int, [ctypes.POINTER(MhaArgs), ctypes.POINTER(MhaPlan)]),
     "llmi_hip_mha_decode": (ctypes.c_int, [ctypes.POINTER(MhaArgs)]),
+    "llmi_hip_mha_decode_static": (ctypes.c_int, [ctypes.POINTER(MhaArgs)]),
     "llmi_hip_mha_decode_append": (ctypes.c_int, [ctypes.POINTER(MhaAppendArgs)]),
     "llmi_hip_mha_workspace_bytes": (c_size_t, [c_i32, c_i32, c_i32]),
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),

@@ -195,6 +195,29 @@ int llmi_hip_mha_decode(const llmi_mha_args* args) {
     return launch_mha_decode(*args, plan);
 }
 
+int llmi_hip_mha_decode_static(const llmi_mha_args* args) {
+    if (!args) return LLMI_ERR_NULL_POINTER;
+    // Plan first, against the size of the static scratch and a stand-in address: an argument or size error
+    // comes back before anything touches the device.
+    llmi_mha_args a = *args;
+    a.workspace = reinterpret_cast<void*>(uintptr_t{256});
+    a.workspace_bytes = LLMI_STATIC_SCRATCH_BYTES;
+    llmi_mha_plan plan;
+    if (int rc = make_plan(&a, &plan)) {
+        if (rc == LLMI_ERR_WORKSPACE)
+            g_last_error = "llmi_hip_mha_decode_static: this head count / split count needs more than the " +
+                           std::to_string(LLMI_STATIC_SCRATCH_BYTES) + "-byte static workspace; use llmi_hip_mha_decode";
+        return rc;
+    }
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    if (int rc = static_scratch(&ptr, &bytes)) return rc;
+    if (plan.workspace_needed > bytes) return LLMI_ERR_WORKSPACE;  // (make_plan has checked this already)
+    a.workspace = ptr;
+    a.workspace_bytes = bytes;
+    return launch_mha_decode(a, plan);
+}
+
 int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
     if (!args) return LLMI_ERR_NULL_POINTER;
     if (!args->key_new || !args->value_new || !args->norm_weight || !args->sin_cache || !args->cos_cache)

@@ -24,6 +24,11 @@ unsigned long long next_epoch();
 // equals a cleared record (all zero) whatever the epoch counter reads -- also when its low bits wrap
 // to zero; the low 31 bits are the epoch's.
 constexpr uint32_t record_tag(unsigned long long epoch) { return 0x80000000u | (uint32_t)(epoch & 0x7fffffffull); }
+// The workspace llmi_hip_mha_decode_static uses instead of a caller's: a fixed array in device memory that
+// belongs to the library's code object (one copy per GPU). static_scratch() returns its address on the
+// current device and its size; it allocates nothing.
+#define LLMI_STATIC_SCRATCH_BYTES (4u << 20)
+int static_scratch(void** ptr, size_t* bytes);
 // Waits of the fused combine that gave up since the library was loaded (device counter of the current device).
 int read_poll_timeouts(unsigned long long* count);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.

@@ -47,10 +47,17 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "llmi_internal.h"
 #include "wave_ops.h"
+
+// Split workspace of llmi_hip_mha_decode_static, for callers that cannot allocate: part of the code
+// object, so every GPU the library runs on holds its own copy from the moment the code object is loaded
+// there until the process ends. In host code the name below only stands for the symbol; the
+// device address comes from hipGetSymbolAddress (static_scratch() below), once per device.
+static __device__ __align__(256) unsigned char scratch[LLMI_STATIC_SCRATCH_BYTES];
 
 namespace llmi {
 
@@ -1005,6 +1012,26 @@ bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipSt
 }
 
 }  // namespace
+
+int static_scratch(void** ptr, size_t* bytes) {
+    // One address per device, looked up with that device current the first time it is asked for.
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* addr[kMaxDevices] = {};
+    int dev = 0;
+    if (int rc = record_hip_error(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= kMaxDevices) return LLMI_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void* p = nullptr;
+        if (int rc = record_hip_error(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+        if (!p) return LLMI_ERR_LAUNCH;
+        addr[dev] = p;
+    }
+    *ptr = addr[dev];
+    *bytes = sizeof(scratch);
+    return LLMI_OK;
+}
 
 int read_poll_timeouts(unsigned long long* count) {
     unsigned int n = 0;
