@@ -63,21 +63,33 @@ def make_arena(torch, dev, ctx_list, n_q=N_Q):
     return k, v, q, regions
 
 
+def kernel_source_blob():
+    """git's blob id of the decode kernel's source (what `git rev-parse HEAD:llminfer_amd/csrc/mha_decode.hip`
+    prints for a committed file), computed from the file itself."""
+    import hashlib
+    data = open(os.path.join(ROOT, "llminfer_amd", "csrc", "mha_decode.hip"), "rb").read()
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+
+
 def measured_traffic(ctx_list):
     """HBM bytes per launch of the decode kernel over the default sweep, as counted by rocprofv3
     (FETCH_SIZE + WRITE_SIZE, each scaled by a calibration copy): bench.py cannot run the profiler on
-    itself, so it reports the figure of the committed counter summary, and only for the workload that
-    summary was taken on."""
+    itself, so it reports the figure of the committed counter summary -- only for the workload that
+    summary was taken on, and only while the kernel source is the one it was taken from (the summary
+    names its git blob id); otherwise None."""
     if ctx_list != DEFAULT_CTX:
         return None
     path = os.path.join(ROOT, "profiles", "mha_decode_kernel_qwen3-4b_ctx1k-32k_hbm_counters.md")
+    traffic = blob = None
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1])
+                traffic = int(line.split(":")[1])
+            if line.startswith("kernel_source_blob:"):
+                blob = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None
+        return None
+    return traffic if blob == kernel_source_blob() else None
 
 
 def cpu_baseline(ctx_list, budget_s=12.0, n_q=N_Q):
@@ -193,8 +205,9 @@ def run_gemv(args):
     return 0
 
 
-def run_stack(args, ctx):
-    """The attention part of a 36-layer decode step at a fixed position, as one HIP graph."""
+def stack_result(args, ctx):
+    """The attention part of a 36-layer decode step at a fixed position, as one HIP graph. `args` needs
+    stack, heads, layout, stack_mode, stack_follow_pos, steps, warmup. Returns the JSON object (or None)."""
     import numpy as np
     from llminfer_amd import _binding as B
     from llminfer_amd import synth
@@ -213,7 +226,7 @@ def run_stack(args, ctx):
     st = host.llmi_host_stack_create(layers, msl, n_q, N_KV, args.layout)
     if not st:
         print("bench.py: " + host.llmi_host_last_error().decode(), file=sys.stderr)
-        return 1
+        return None
 
     def up(ptr, arr):
         arr = np.ascontiguousarray(arr)
@@ -271,7 +284,7 @@ def run_stack(args, ctx):
         per_layer += ((n_q * HEAD_DIM + 2 * KV_DIM) * hidden + hidden * n_q * HEAD_DIM) * 2 + 3 * hidden * 2
     gbs = layers * per_layer / (us_token * 1e-6) / 1e9
     host.llmi_host_stack_destroy(st)
-    print(json.dumps({
+    return {
         "metric": "attention stack of one decode step, us per token", "value": round(us_token, 2), "unit": "us/token",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us_token / 1e3, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -285,7 +298,198 @@ def run_stack(args, ctx):
         "us_per_layer": round(us_token / layers, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
-    }))
+    }
+
+
+def run_stack(args, ctx):
+    res = stack_result(args, ctx)
+    if res is None:
+        return 1
+    print(json.dumps(res))
+    return 0
+
+
+class Sweep:
+    """Decode-attention calls over rotating KV slices, captured into HIP graphs and timed with HIP events."""
+
+    def __init__(self, ctx_list, n_q=N_Q, layout=1):
+        import torch
+        from llminfer_amd import _binding as B
+        from llminfer_amd import ops
+        self.torch, self.B, self.ops = torch, B, ops
+        self.ctx_list, self.n_q, self.layout = list(ctx_list), n_q, layout
+        self.dev = torch.device("cuda:0")
+        self.k, self.v, self.q, self.regions = make_arena(torch, self.dev, self.ctx_list, n_q)
+        self.out = torch.empty(n_q * HEAD_DIM, dtype=torch.bfloat16, device=self.dev)
+        self.ws = torch.empty(ops.workspace_bytes(n_q, HEAD_DIM, max(self.ctx_list)) // 4, dtype=torch.float32, device=self.dev)
+        self.sink = torch.zeros(64, dtype=torch.int32, device=self.dev)
+        self.stream = torch.cuda.Stream()
+        self.decode = B.lib().llmi_hip_mha_decode
+
+    def call_args(self, ctx, s, **over):
+        off = self.regions[(ctx, s)] * 2
+        return self.ops.make_mha_args(self.q, self.k.data_ptr() + off, self.v.data_ptr() + off, self.out, self.ws, layer_id=0,
+                                      pos=ctx - 1, kv_dim=KV_DIM, kv_mul=self.n_q // N_KV, head_num=self.n_q, head_dim=HEAD_DIM,
+                                      max_seq_len=ctx, kv_layout=self.layout, **over)
+
+    def plan(self, ctx, **over):
+        return self.ops.mha_plan(self.call_args(ctx, 0, **over))
+
+    def enqueue(self, ctxs, first_step, steps, **over):
+        """Steps first_step .. first_step+steps-1: one call per context each, on slice step % SLICES."""
+        for s in range(first_step, first_step + steps):
+            for ctx in ctxs:
+                a = self.call_args(ctx, s % SLICES, **over)
+                a.stream = self.stream.cuda_stream
+                self.B.check(self.decode(ctypes.byref(a)), "llmi_hip_mha_decode")
+
+    def enqueue_floor(self, ctxs, first_step, steps, workgroups, waves, inflight):
+        probe = self.B.lib().llmi_hip_probe_stream_read
+        for s in range(first_step, first_step + steps):
+            for ctx in ctxs:
+                off = self.regions[(ctx, s % SLICES)] * 2
+                self.B.check(probe(self.k.data_ptr() + off, self.v.data_ptr() + off, ctx * KV_DIM * 2, workgroups, waves,
+                                   inflight, self.sink.data_ptr(), self.stream.cuda_stream), "llmi_hip_probe_stream_read")
+
+    def capture(self, enqueue_fn, steps=SLICES):
+        """A graph of `steps` steps (eager once first: loads the code objects before capture)."""
+        torch = self.torch
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(self.stream):
+            enqueue_fn(0, 1)
+            self.stream.synchronize()
+            with torch.cuda.graph(g, stream=self.stream):
+                enqueue_fn(0, steps)
+        return g
+
+    def time_replays(self, graphs_and_counts):
+        """Elapsed ms of the given replays, in order, between two events on the replaying stream."""
+        torch = self.torch
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(self.stream):
+            e0.record(self.stream)
+            for g, n in graphs_and_counts:
+                for _ in range(n):
+                    g.replay()
+            e1.record(self.stream)
+        e1.synchronize()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1)
+
+    def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None):
+        """Best of `reps` batches of graph replays, us per call."""
+        g = self.capture(enqueue_fn)
+        self.time_replays([(g, 8)])
+        n = replays or 40
+        best = min(self.time_replays([(g, n)]) for _ in range(reps))
+        return best * 1e3 / (n * SLICES * calls_per_step)
+
+
+# stream-only configurations tried for the floor: (workgroups, waves per workgroup, tiles in flight per wave)
+FLOOR_CONFIGS = [(256, 4, 2), (256, 8, 2), (512, 4, 2), (256, 4, 4), (512, 8, 1), (1024, 4, 1), (512, 4, 4), (256, 8, 4)]
+
+
+def stream_floor(sw, ctx_list, configs=FLOOR_CONFIGS):
+    """Per context: the fastest stream-only launch (same K/V bytes read once and thrown away, same graph-replay
+    timing as the decode figures) over a handful of launch shapes."""
+    rows = []
+    for ctx in ctx_list:
+        best = None
+        for wg, waves, inflight in configs:
+            tiles = ctx * KV_DIM * 2 // 4096
+            if wg > tiles:
+                continue
+            us = sw.us_per_call(lambda f, n: sw.enqueue_floor([ctx], f, n, wg, waves, inflight), reps=2)
+            if best is None or us < best[0]:
+                best = (us, wg, waves, inflight)
+        us, wg, waves, inflight = best
+        gbs = 2 * ctx * KV_DIM * 2 / (us * 1e-6) / 1e9
+        rows.append({"ctx": ctx, "us": round(us, 3), "GBps": round(gbs, 1), "frac_peak": round(gbs / HBM_PEAK_GBS, 4),
+                     "workgroups": wg, "waves": waves, "tiles_in_flight": inflight})
+    return rows
+
+
+DISPATCH_CTX = [96, 160, 176, 300, 700, 1024, 1500, 3000, 4097, 5000, 9000, 12345, 20000, 32768]
+
+
+def dispatch_rows(sw, ctx_list):
+    """What the dispatcher picks against forced alternatives, per context length: single pass, and the fused
+    split path at several split counts; same timing method as the per-context figures."""
+    B = sw.B
+    rows = []
+    for ctx in ctx_list:
+        def timed(**over):
+            return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over))
+        if not rows:
+            timed()  # the first graph timed in a process runs 1-2 us per call slow: discard one
+        auto = timed()
+        alts = {}
+        if ctx <= 1024:
+            alts["single"] = timed(force_path=B.PATH_SINGLE_PASS)
+        tiles = (ctx + 15) // 16
+        for sp in (4, 8, 16, 32, 64):
+            if sp <= tiles:
+                alts["split%d" % sp] = timed(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
+        best = min(alts, key=alts.get)
+        p = sw.plan(ctx)
+        rows.append({"ctx": ctx, "auto_us": round(auto, 2), "auto_plan": "path%d S=%d W=%d" % (p.path, p.num_splits, p.waves_per_group),
+                     "best_forced": best, "best_forced_us": round(alts[best], 2), "auto_over_best": round(auto / alts[best], 3),
+                     "forced_us": {k2: round(v2, 2) for k2, v2 in alts.items()}})
+    return rows
+
+
+def per_ctx_rows(sw, ctx_list, replays):
+    rows = []
+    for ctx in ctx_list:
+        us = sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n), reps=3, replays=replays)
+        gbs = algorithmic_bytes(ctx, sw.n_q) / (us * 1e-6) / 1e9
+        p = sw.plan(ctx)
+        rows.append({"ctx": ctx, "us_per_layer": round(us, 3), "GBps": round(gbs, 1), "frac_peak": round(gbs / HBM_PEAK_GBS, 4),
+                     "path": p.path, "splits": p.num_splits, "waves": p.waves_per_group})
+    return rows
+
+
+def run_calibrate_hbm(args):
+    """A plain copy kernel of known traffic, for scaling the FETCH_SIZE / WRITE_SIZE counters:
+    rocprofv3 --pmc FETCH_SIZE --kernel-trace -- python3 bench.py --calibrate-hbm"""
+    import torch
+    from llminfer_amd import _binding as B
+    gib = 1 << 30
+    src = torch.ones(gib // 4, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(6):
+        B.check(B.lib().llmi_hip_probe_copy(src.data_ptr(), dst.data_ptr(), gib, torch.cuda.current_stream().cuda_stream), "copy")
+    torch.cuda.synchronize()
+    print(json.dumps({"metric": "calibration copy", "kernel": "copy_kernel", "dispatches": 6, "bytes_read_per_dispatch": gib,
+                      "bytes_written_per_dispatch": gib, "ok": bool(torch.equal(src[:1024], dst[:1024]))}))
+    return 0
+
+
+def run_handover_probe(args):
+    """How a 4-byte value stored by one workgroup becomes visible to a polling workgroup on the same XCD and
+    on another one, for every pair of store / load cache policies."""
+    import torch
+    from llminfer_amd import _binding as B
+    names = ["plain", "sc0", "sc1", "sc0 sc1", "nt"]
+    line = torch.zeros(1024, dtype=torch.int32, device="cuda:0")
+    res_d = torch.zeros(8, dtype=torch.int32, device="cuda:0")
+    rows = []
+    for place, reader in (("same XCD", 8), ("next XCD", 9)):
+        for precache in (1, 0):
+            for st in range(5):
+                for ld in range(5):
+                    reps = []
+                    for _ in range(3):
+                        B.check(B.lib().llmi_hip_probe_handover(st, ld, reader, precache, line.data_ptr(), res_d.data_ptr(),
+                                                               torch.cuda.current_stream().cuda_stream), "handover probe")
+                        torch.cuda.synchronize()
+                        r = res_d.cpu().numpy()
+                        reps.append({"seen": int(r[0]), "polls": int(r[1]), "ns": int(r[2]), "xcc_reader": int(r[3]), "xcc_writer": int(r[4])})
+                    rows.append({"placement": place, "precache": precache, "store": names[st], "load": names[ld], "runs": reps})
+    print(json.dumps({"metric": "hand-over probe: store policy x load policy, reader polls until it sees the writer's value "
+                                "(writer waits 2 us before storing; 4000 polls at most)", "rows": rows}))
     return 0
 
 
@@ -296,8 +500,15 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--ctx", type=str, default=",".join(map(str, DEFAULT_CTX)))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="headline sweep only: skip the stream floor, the position-major layout, BASELINE configs 4 and 5 "
+                         "and the dispatch check that the default run appends to its JSON line")
     ap.add_argument("--dispatch-check", action="store_true",
                     help="time the automatic plan against forced single-pass / split plans at every --ctx")
+    ap.add_argument("--stream-floor", action="store_true",
+                    help="time a kernel that only reads the same K/V bytes, next to the decode kernel, at every --ctx")
+    ap.add_argument("--calibrate-hbm", action="store_true", help="run the copy kernel of known traffic (for rocprofv3 --pmc)")
+    ap.add_argument("--handover-probe", action="store_true", help="store/load cache-policy visibility probe between two workgroups")
     ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
     ap.add_argument("--heads", type=int, default=N_Q, help="query heads (32 = Qwen3-4B, 64 = Qwen3-32B head layout)")
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
@@ -316,166 +527,151 @@ def main():
         print("bench.py: this build measures one GPU only (--gpus %d refused): decode attention at batch 1 "
               "has no multi-GPU part here." % args.gpus, file=sys.stderr)
         return 2
+    if args.steps < 1 or args.warmup < 0:
+        print("bench.py: --steps must be positive, --warmup non-negative", file=sys.stderr)
+        return 2
     ctx_list = [int(c) for c in args.ctx.split(",")]
     n_q = args.heads
+
+    import torch
+    from llminfer_amd import _binding as B
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    B.lib()  # fail loudly if the HIP library is not built
+    torch.cuda.set_device(torch.device("cuda:0"))
+
+    if args.calibrate_hbm:
+        return run_calibrate_hbm(args)
+    if args.handover_probe:
+        return run_handover_probe(args)
     if args.gemv:
         return run_gemv(args)
     if args.stack:
         return run_stack(args, ctx_list[0])
 
-    import torch
-    from llminfer_amd import _binding as B
-    from llminfer_amd import ops
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        return 1
-    B.lib()  # fail loudly if the HIP library is not built
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-
-    k, v, q, regions = make_arena(torch, dev, ctx_list, n_q)
-    out = torch.empty(n_q * HEAD_DIM, dtype=torch.bfloat16, device=dev)
-    ws = torch.empty(ops.workspace_bytes(n_q, HEAD_DIM, max(ctx_list)) // 4, dtype=torch.float32, device=dev)
-    esz = 2
-
-    def call_args(ctx, s, **over):
-        off = regions[(ctx, s)] * esz
-        return ops.make_mha_args(q, k.data_ptr() + off, v.data_ptr() + off, out, ws, layer_id=0, pos=ctx - 1,
-                                 kv_dim=KV_DIM, kv_mul=n_q // N_KV, head_num=n_q, head_dim=HEAD_DIM,
-                                 max_seq_len=ctx, kv_layout=args.layout, **over)
-
-    plans = {ctx: ops.mha_plan(call_args(ctx, 0)) for ctx in ctx_list}
-    stream = torch.cuda.Stream()
-    decode = B.lib().llmi_hip_mha_decode
-
-    def enqueue(ctxs, steps, **over):
-        for s in range(steps):
-            for ctx in ctxs:
-                a = call_args(ctx, s % SLICES, **over)
-                a.stream = stream.cuda_stream
-                B.check(decode(ctypes.byref(a)), "llmi_hip_mha_decode")
-
-    def capture(ctxs, **over):
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(stream):
-            enqueue(ctxs, 1, **over)  # eager once: loads the code objects before capture
-            stream.synchronize()
-            with torch.cuda.graph(g, stream=stream):
-                enqueue(ctxs, SLICES, **over)
-        return g
-
-    def time_graph(g, replays):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        with torch.cuda.stream(stream):
-            e0.record(stream)
-            for _ in range(replays):
-                g.replay()
-            e1.record(stream)
-        e1.synchronize()
-        return e0.elapsed_time(e1)  # ms
+    sw = Sweep(ctx_list, n_q, args.layout)
+    layout_name = "head-major" if args.layout == 1 else "position-major"
 
     if args.dispatch_check:
-        # What the dispatcher picks against forced alternatives, per context length: single pass, and the
-        # fused split path at several split counts (4 waves); same timing method as the per-context figures.
-        rows = []
-        for ctx in ctx_list:
-            def timed(**over):
-                g = capture([ctx], **over)
-                time_graph(g, 8)
-                torch.cuda.synchronize()
-                n = max(SLICES, args.steps // 4 // SLICES * SLICES)
-                best_ms = None
-                for _ in range(3):  # best of three batches: a batch now and then runs 1-2 us per call slow
-                    t = time_graph(g, n // SLICES)
-                    torch.cuda.synchronize()
-                    best_ms = t if best_ms is None else min(best_ms, t)
-                return best_ms * 1e3 / n
-            if not rows:
-                timed()  # the first graph timed in a process runs 1-2 us per call slow: discard one
-            auto = timed()
-            alts = {}
-            if ctx <= 1024:
-                alts["single"] = timed(force_path=B.PATH_SINGLE_PASS)
-            tiles = (ctx + 15) // 16
-            for sp in (4, 8, 16, 32, 64):
-                if sp <= tiles:
-                    alts["split%d" % sp] = timed(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
-            best = min(alts, key=alts.get)
-            p = plans[ctx]
-            rows.append({"ctx": ctx, "auto_us": round(auto, 2), "auto_plan": "path%d S=%d W=%d" % (p.path, p.num_splits, p.waves_per_group),
-                         "best_forced": best, "best_forced_us": round(alts[best], 2),
-                         "auto_over_best": round(auto / alts[best], 3),
-                         "forced_us": {k2: round(v2, 2) for k2, v2 in alts.items()}})
+        rows = dispatch_rows(sw, ctx_list)
         print(json.dumps({"metric": "dispatch check: auto plan against forced paths, us per layer call", "n_gpus": 1,
-                          "config": {"workload": "%d Q / 8 KV heads, %s layout" % (n_q, "head-major" if args.layout == 1 else "position-major")},
+                          "config": {"workload": "%d Q / 8 KV heads, %s layout" % (n_q, layout_name)},
                           "rows": rows, "worst_auto_over_best": max(r["auto_over_best"] for r in rows)}))
         return 0
+    if args.stream_floor:
+        floor = stream_floor(sw, ctx_list)
+        mine = per_ctx_rows(sw, ctx_list, 40)
+        rows = [dict(f, decode_us=m["us_per_layer"], decode_frac_peak=m["frac_peak"], decode_minus_floor_us=round(m["us_per_layer"] - f["us"], 3))
+                for f, m in zip(floor, mine)]
+        print(json.dumps({"metric": "stream-only floor next to the decode kernel, us per launch (graph replays)", "n_gpus": 1,
+                          "config": {"workload": "K and V rows of one call (%d Q / 8 KV heads, %s) read once and thrown away; best of %d "
+                                                 "launch shapes" % (n_q, layout_name, len(FLOOR_CONFIGS))},
+                          "rows": rows}))
+        return 0
 
-    # ---- the timed region: K steps of the whole sweep ----------------------
-    steps = max(SLICES, (args.steps + SLICES - 1) // SLICES * SLICES)
-    warm = max(SLICES, (args.warmup + SLICES - 1) // SLICES * SLICES)
-    g_all = capture(ctx_list)
-    time_graph(g_all, warm // SLICES)
-    torch.cuda.synchronize()
-    ms = time_graph(g_all, steps // SLICES)
-    torch.cuda.synchronize()
+    # ---- the timed region: EXACTLY --steps steps of the whole sweep, after --warmup untimed ones ----------
+    # A graph holds SLICES steps (one per KV slice); a second, shorter graph holds the remainder.
+    def sweep_enqueue(first, n):
+        sw.enqueue(ctx_list, first, n)
+
+    g_full = sw.capture(sweep_enqueue, SLICES)
+    rem_graphs = {}
+
+    def replays_for(k):
+        full, rem = divmod(k, SLICES)
+        seq = [(g_full, full)] if full else []
+        if rem:
+            if rem not in rem_graphs:
+                rem_graphs[rem] = sw.capture(sweep_enqueue, rem)
+            seq.append((rem_graphs[rem], 1))
+        return seq
+
+    timed_seq = replays_for(args.steps)  # (captured before the clock starts)
+    if args.warmup:
+        sw.time_replays(replays_for(args.warmup))
+    ms = sw.time_replays(timed_seq)
+    steps = args.steps
     ms_per_step = ms / steps
     step_bytes = sum(algorithmic_bytes(c, n_q) for c in ctx_list)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     launches_per_step = len(ctx_list)  # every call of the sweep is one launch of the decode kernel
 
-    # ---- per-context figures (same method, one context at a time) ----------
-    per_ctx = []
-    for ctx in ctx_list:
-        g = capture([ctx])
-        time_graph(g, max(1, warm // SLICES))
-        torch.cuda.synchronize()
-        n = max(SLICES, steps)
-        t = time_graph(g, n // SLICES)
-        torch.cuda.synchronize()
-        us = t * 1e3 / n
-        # Spread: 32 batches of eight replays each, an event between batches, nothing else on the stream.
-        marks = [torch.cuda.Event(enable_timing=True) for _ in range(33)]
-        with torch.cuda.stream(stream):
-            marks[0].record(stream)
-            for b in range(32):
-                for _ in range(8):
-                    g.replay()
-                marks[b + 1].record(stream)
-        marks[-1].synchronize()
-        batch_us = sorted(marks[b].elapsed_time(marks[b + 1]) * 1e3 / (8 * SLICES) for b in range(32))
-        gbs = algorithmic_bytes(ctx, n_q) / (us * 1e-6) / 1e9
-        p = plans[ctx]
-        per_ctx.append({"ctx": ctx, "us_per_layer": round(us, 3), "us_p10": round(batch_us[3], 3),
-                        "us_median": round(0.5 * (batch_us[15] + batch_us[16]), 3), "us_p90": round(batch_us[28], 3),
-                        "GBps": round(gbs, 1),
-                        "frac_peak": round(gbs / HBM_PEAK_GBS, 4), "path": p.path, "splits": p.num_splits,
-                        "waves": p.waves_per_group})
+    # ---- the same sweep again for at least half a second: median over batches (a short --steps leaves a
+    # timed region of a millisecond or two, which a machine hiccup can move) ---------------------------
+    batch_ms = []
+    t_long = time.perf_counter()
+    while len(batch_ms) < 5 or (time.perf_counter() - t_long < 0.5 and len(batch_ms) < 400):
+        batch_ms.append(sw.time_replays([(g_full, 10)]) / (10 * SLICES))
+    batch_ms.sort()
+    median_ms = batch_ms[len(batch_ms) // 2]
 
+    per_ctx = per_ctx_rows(sw, ctx_list, 40)
     avg_launch_us = ms_per_step * 1e3 / launches_per_step
     avg_launch_bytes = step_bytes / launches_per_step
     achieved = avg_launch_bytes / (avg_launch_us * 1e-6) / 1e9
     result = {
         "metric": "GQA decode attn us/layer + HBM GB/s (% peak), Qwen3-4B shape, ctx 1K-32K",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%s layer shape (%d Q / 8 KV heads, head_dim 128), batch 1, one decode-"
                                "attention layer call per context in %s per step, bf16 KV cache, %s layout, "
                                "HIP-graph replays over %d rotating KV slices per context"
                                % ("Qwen3-4B" if n_q == 32 else "Qwen3-32B-heads" if n_q == 64 else "custom", n_q,
-                                  ctx_list, "head-major" if args.layout == 1 else "position-major", SLICES),
+                                  ctx_list, layout_name, SLICES),
                    "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout},
+        "timed_region_s": round(ms * 1e-3, 6),
+        "long_run": {"seconds": round(sum(batch_ms) * 10 * SLICES * 1e-3, 3), "batches": len(batch_ms), "steps_per_batch": 10 * SLICES,
+                     "ms_per_step_median": round(median_ms, 6), "value_median": round(step_bytes / (median_ms * 1e-3) / 1e9, 1),
+                     "ms_per_step_p10": round(batch_ms[len(batch_ms) // 10], 6), "ms_per_step_p90": round(batch_ms[len(batch_ms) * 9 // 10], 6)},
         "us_per_layer_mean": round(avg_launch_us, 3),
         "per_ctx": per_ctx,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic(ctx_list) if n_q == N_Q else None,
+                     "traffic": measured_traffic(ctx_list) if n_q == N_Q and args.layout == 1 else None,
                      "kernel": "mha_decode_kernel", "launches": steps * launches_per_step,
                      "avg_launch_us": round(avg_launch_us, 3), "avg_launch_bytes": int(avg_launch_bytes)},
     }
+
+    if not args.no_extras:
+        # What one launch can reach on this machine with the same bytes: the stream-only floor per context.
+        floor = stream_floor(sw, ctx_list)
+        for row, f in zip(per_ctx, floor):
+            row["stream_floor_us"] = f["us"]
+            row["stream_floor_frac_peak"] = f["frac_peak"]
+        result["stream_floor"] = floor
+        del sw
+        torch.cuda.empty_cache()
+        if n_q == N_Q and args.layout == 1:
+            # the reference's own cache layout (what a maintainer gets who changes nothing but the registry arm)
+            sw_pm = Sweep(ctx_list, n_q, 0)
+            result["position_major"] = per_ctx_rows(sw_pm, ctx_list, 40)
+            del sw_pm
+            torch.cuda.empty_cache()
+            # the dispatch against forced plans at lengths either side of the threshold, powers of two and not
+            sw_d = Sweep(DISPATCH_CTX, n_q, 1)
+            rows = dispatch_rows(sw_d, DISPATCH_CTX)
+            result["dispatch_check"] = {"worst_auto_over_best": max(r["auto_over_best"] for r in rows),
+                                        "rows": [{k2: r[k2] for k2 in ("ctx", "auto_us", "auto_plan", "best_forced", "best_forced_us", "auto_over_best")}
+                                                 for r in rows]}
+            del sw_d
+            torch.cuda.empty_cache()
+            # BASELINE config 5: 64 Q / 8 KV heads at ctx 131072 (512 MiB of K and V per call)
+            sw5 = Sweep([131072], 64, 1)
+            r5 = per_ctx_rows(sw5, [131072], 10)[0]
+            f5 = stream_floor(sw5, [131072], FLOOR_CONFIGS[:4])[0]
+            result["cfg5"] = dict(r5, workload="64 Q / 8 KV heads, ctx 131072, head-major, graph replays over %d KV slices" % SLICES,
+                                  stream_floor_us=f5["us"])
+            del sw5
+            torch.cuda.empty_cache()
+            # BASELINE config 4: 36 layers at ctx 4096 + 1 new token, fused QK-Norm + RoPE + append, one HIP graph per token
+            ns = argparse.Namespace(stack=36, heads=32, layout=1, stack_mode=2, stack_follow_pos=False, steps=200, warmup=20)
+            r4 = stack_result(ns, 4096)
+            if r4 is not None:
+                result["cfg4_stack"] = {"us_per_token": r4["value"], "us_per_layer": r4["us_per_layer"],
+                                        "frac_peak": r4["roofline"]["frac"], "GBps": r4["roofline"]["achieved"],
+                                        "workload": r4["config"]["workload"]}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(ctx_list, n_q=n_q)
     print(json.dumps(result))

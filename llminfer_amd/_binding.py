@@ -77,6 +77,10 @@ class QkNormRopeArgs(ctypes.Structure):
     ]
 
 
+class ProbeHandoverResult(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint32) for n in ("seen", "polls", "ns", "xcc_reader", "xcc_writer")]
+
+
 class PoolStats(ctypes.Structure):
     _fields_ = [(n, c_size_t) for n in (
         "backing_allocs", "reuses", "big_busy_blocks", "big_free_blocks", "small_busy_blocks",
@@ -113,6 +117,10 @@ SYMBOLS = {
     "llmi_hip_abi_version": (ctypes.c_int, []),
     "llmi_hip_set_poll_limit": (c_i32, [c_i32]),
     "llmi_hip_poll_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint64)]),
+    # include/llmi_hip_probes.h
+    "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
+    "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
 }

@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libllmi_hip.so")
 HOST_LIB_PATH = os.path.join(HERE, "libllmi_host.so")
 
-HIP_SOURCES = ["mha_decode.hip", "qk_norm_rope.hip", "gemv.hip", "c_api.cpp", "pool.cpp"]
+HIP_SOURCES = ["mha_decode.hip", "qk_norm_rope.hip", "gemv.hip", "probes.hip", "c_api.cpp", "pool.cpp"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops.
 HIPCC_FLAGS = [

@@ -1,0 +1,196 @@
+// Measurement kernels (declared in llmi_hip_probes.h): a stream-only reader with the decode kernel's
+// access pattern, a plain copy of known traffic, and a two-workgroup hand-over probe. Nothing here
+// is on the product path.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "llmi_hip_probes.h"
+#include "llmi_internal.h"
+
+namespace llmi {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Workgroup g reads tiles [g*T/G, (g+1)*T/G) of both arrays (T tiles of 4 KiB each); its wavefronts take
+// the tiles of that run in turn, INFLIGHT tiles of each array requested before the first is consumed.
+template <int NW, int INFLIGHT>
+__global__ __launch_bounds__(NW * 64) void stream_read_kernel(const char* __restrict__ a, const char* __restrict__ b,
+                                                              uint32_t tiles, uint32_t* sink) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t g = blockIdx.x, G = gridDim.x;
+    const uint32_t run = tiles / G, longer = tiles % G;
+    const uint32_t first = g * run + (g < longer ? g : longer);
+    const uint32_t count = run + (g < longer ? 1u : 0u);
+    const char* pa = a + (size_t)first * 4096u + lane * 16u;
+    const char* pb = b + (size_t)first * 4096u + lane * 16u;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (uint32_t t0 = wave; t0 < count; t0 += NW * INFLIGHT) {
+        u32x4 r[INFLIGHT][8];
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+            uint32_t t = t0 + u * NW;
+            if (t >= count) t = t0;  // (a repeat near the end of the run: served by the cache, never out of range)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                r[u][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pa + (size_t)t * 4096u + j * 1024u));
+                r[u][4 + j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pb + (size_t)t * 4096u + j * 1024u));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc ^= r[u][j];
+    }
+    // Keeps the loads alive; the condition does not hold for any data a benchmark feeds it.
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[0] = acc[0];
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+__device__ __forceinline__ uint32_t xcc_id() {
+    uint32_t x;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+    return x & 15u;
+}
+
+template <int M>
+__device__ __forceinline__ uint32_t load_policy(const uint32_t* p) {
+    uint32_t v;
+    if constexpr (M == LLMI_PROBE_PLAIN) asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    if constexpr (M == LLMI_PROBE_SC0) asm volatile("global_load_dword %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    if constexpr (M == LLMI_PROBE_SC1) asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    if constexpr (M == LLMI_PROBE_SC0_SC1) asm volatile("global_load_dword %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    if constexpr (M == LLMI_PROBE_NT) asm volatile("global_load_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int M>
+__device__ __forceinline__ void store_policy(uint32_t* p, uint32_t v) {
+    if constexpr (M == LLMI_PROBE_PLAIN) asm volatile("global_store_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    if constexpr (M == LLMI_PROBE_SC0) asm volatile("global_store_dword %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    if constexpr (M == LLMI_PROBE_SC1) asm volatile("global_store_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    if constexpr (M == LLMI_PROBE_SC0_SC1) asm volatile("global_store_dword %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    if constexpr (M == LLMI_PROBE_NT) asm volatile("global_store_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+}
+
+constexpr uint32_t kProbeValue = 42u;
+constexpr uint32_t kProbePolls = 4000u;
+
+// line[0]: the data word; line[64] (another 256-byte line): reader -> writer "I am polling".
+template <int WM, int RM>
+__global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe_handover_result* res, int reader_wg, int precache) {
+    if (threadIdx.x != 0) return;
+    uint32_t* data = line;
+    uint32_t* flag = line + 64;
+    if ((int)blockIdx.x == reader_wg) {
+        if (precache) (void)(load_policy<LLMI_PROBE_PLAIN>(data) + load_policy<RM>(data));
+        store_policy<LLMI_PROBE_SC1>(flag, 1u);
+        const unsigned long long t0 = wall_clock64();
+        uint32_t polls = 0, seen = 0;
+        for (; polls < kProbePolls; ++polls)
+            if (load_policy<RM>(data) == kProbeValue) {
+                seen = 1;
+                break;
+            }
+        const unsigned long long t1 = wall_clock64();
+        res->seen = seen;
+        res->polls = polls;
+        res->ns = (uint32_t)((t1 - t0) * 10ull);
+        res->xcc_reader = xcc_id();
+    } else if (blockIdx.x == 0) {
+        res->xcc_writer = xcc_id();
+        for (int i = 0; i < 200000; ++i)  // bounded: the reader raises the flag at once
+            if (load_policy<LLMI_PROBE_SC1>(flag) == 1u) break;
+        const unsigned long long t0 = wall_clock64();
+        while (wall_clock64() - t0 < 200ull) {  // 2 us: the reader is polling by now
+        }
+        store_policy<WM>(data, kProbeValue);
+    }
+}
+
+typedef void (*HandoverKernel)(uint32_t*, llmi_probe_handover_result*, int, int);
+template <int WM>
+HandoverKernel pick_reader(int rm) {
+    switch (rm) {
+        case LLMI_PROBE_PLAIN: return handover_kernel<WM, LLMI_PROBE_PLAIN>;
+        case LLMI_PROBE_SC0: return handover_kernel<WM, LLMI_PROBE_SC0>;
+        case LLMI_PROBE_SC1: return handover_kernel<WM, LLMI_PROBE_SC1>;
+        case LLMI_PROBE_SC0_SC1: return handover_kernel<WM, LLMI_PROBE_SC0_SC1>;
+        default: return handover_kernel<WM, LLMI_PROBE_NT>;
+    }
+}
+
+template <int NW>
+bool launch_stream(int inflight, dim3 grid, hipStream_t s, const char* a, const char* b, uint32_t tiles, uint32_t* sink) {
+    switch (inflight) {
+        case 1: hipLaunchKernelGGL((stream_read_kernel<NW, 1>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
+        case 2: hipLaunchKernelGGL((stream_read_kernel<NW, 2>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
+        case 4: hipLaunchKernelGGL((stream_read_kernel<NW, 4>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
+        default: return false;
+    }
+}
+
+}  // namespace
+}  // namespace llmi
+
+using namespace llmi;
+
+extern "C" {
+
+int llmi_hip_probe_stream_read(const void* a, const void* b, size_t bytes_each, int32_t workgroups, int32_t waves,
+                               int32_t tiles_in_flight, void* sink, void* stream) {
+    if (!a || !b || !sink) return LLMI_ERR_NULL_POINTER;
+    if (bytes_each == 0 || bytes_each % 4096 != 0 || bytes_each / 4096 > 0xffffffffull) return LLMI_ERR_INVALID_ARG;
+    if (workgroups < 1 || workgroups > 65535) return LLMI_ERR_INVALID_ARG;
+    if (((uintptr_t)a | (uintptr_t)b) & 15u) return LLMI_ERR_ALIGNMENT;
+    const uint32_t tiles = (uint32_t)(bytes_each / 4096);
+    const char* pa = static_cast<const char*>(a);
+    const char* pb = static_cast<const char*>(b);
+    uint32_t* ps = static_cast<uint32_t*>(sink);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    bool ok = false;
+    switch (waves) {
+        case 1: ok = launch_stream<1>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
+        case 2: ok = launch_stream<2>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
+        case 4: ok = launch_stream<4>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
+        case 8: ok = launch_stream<8>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
+        default: ok = false;
+    }
+    if (!ok) return LLMI_ERR_INVALID_ARG;
+    return check_launch();
+}
+
+int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream) {
+    if (!src || !dst) return LLMI_ERR_NULL_POINTER;
+    if (bytes == 0 || bytes % 16 != 0) return LLMI_ERR_INVALID_ARG;
+    if (((uintptr_t)src | (uintptr_t)dst) & 15u) return LLMI_ERR_ALIGNMENT;
+    hipLaunchKernelGGL(copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), bytes / 16);
+    return check_launch();
+}
+
+int llmi_hip_probe_handover(int32_t store_pol, int32_t load_pol, int32_t reader_workgroup, int32_t precache, void* line,
+                            llmi_probe_handover_result* result, void* stream) {
+    if (!line || !result) return LLMI_ERR_NULL_POINTER;
+    if (store_pol < 0 || store_pol > LLMI_PROBE_NT || load_pol < 0 || load_pol > LLMI_PROBE_NT) return LLMI_ERR_INVALID_ARG;
+    if (reader_workgroup < 1 || reader_workgroup > 15) return LLMI_ERR_INVALID_ARG;
+    if ((uintptr_t)line & 255u) return LLMI_ERR_ALIGNMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = record_hip_error(hipMemsetAsync(line, 0, 4096, s), "hipMemsetAsync")) return rc;
+    if (int rc = record_hip_error(hipMemsetAsync(result, 0, sizeof(*result), s), "hipMemsetAsync")) return rc;
+    HandoverKernel k;
+    switch (store_pol) {
+        case LLMI_PROBE_PLAIN: k = pick_reader<LLMI_PROBE_PLAIN>(load_pol); break;
+        case LLMI_PROBE_SC0: k = pick_reader<LLMI_PROBE_SC0>(load_pol); break;
+        case LLMI_PROBE_SC1: k = pick_reader<LLMI_PROBE_SC1>(load_pol); break;
+        case LLMI_PROBE_SC0_SC1: k = pick_reader<LLMI_PROBE_SC0_SC1>(load_pol); break;
+        default: k = pick_reader<LLMI_PROBE_NT>(load_pol); break;
+    }
+    hipLaunchKernelGGL(k, dim3(16), dim3(64), 0, s, static_cast<uint32_t*>(line), result, (int)reader_workgroup, (int)precache);
+    return check_launch();
+}
+
+}  // extern "C"

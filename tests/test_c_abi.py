@@ -12,11 +12,11 @@ import pytest
 from llminfer_amd import _binding as B
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "llmi_hip.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("llmi_hip.h", "llmi_hip_probes.h")]
 
 
 def declared_functions():
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b(llmi_[a-z0-9_]+)\s*\(", text)
     # typedef'd function-pointer types are not exported symbols
