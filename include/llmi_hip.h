@@ -155,7 +155,7 @@ typedef struct llmi_mha_append_args {
  * are stored to the cache (either layout) and used from registers. The normalised query is not written
  * back. Replaces the back-to-back pair fused_qk_norm_rope + mha of the reference's layer loop
  * (code/source/model/qwen3_fused.cpp:524-548; kernels rmsnorm_kernel.cu:248-290, mha_kernel.cu:440-529).
- * The separate-combine path (LLMI_PATH_SPLIT) and 8 waves per workgroup are not available here. */
+ * The separate-combine path (LLMI_PATH_SPLIT) is not available here. */
 int llmi_hip_mha_decode_append(const llmi_mha_append_args* args);
 
 /* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */

@@ -229,10 +229,9 @@ int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
     for (const void* p : ptrs)
         if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
     if (!(args->eps >= 0.0f)) return LLMI_ERR_INVALID_ARG;
-    if (args->mha.force_path == LLMI_PATH_SPLIT || args->mha.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
+    if (args->mha.force_path == LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
     llmi_mha_plan plan;
-    if (int rc = make_plan(&args->mha, &plan, 4, 1)) return rc;
-    if (plan.waves_per_group > 4) return LLMI_ERR_INVALID_ARG;
+    if (int rc = make_plan(&args->mha, &plan, kMaxWaves, 1)) return rc;
     return launch_mha_decode(args->mha, plan, args);
 }
 

@@ -985,10 +985,8 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
         dim3 grid(n_kv, ka.num_splits);
     const bool dyn = ka.pos_dev != nullptr;  // position read at run time: its own instantiation, the static one pays nothing
     if (append) {
-        if constexpr (NW <= 4) {
-            if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
-            else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
-        }
+        if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
     } else {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else if (ka.stagger && ka.num_splits > 1)
@@ -999,7 +997,6 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
 
 template <int G>
 bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream) {
-    if (append && nw > 4) return false;
     switch (nw) {
         case 1: launch_decode<G, 1>(ka, n_kv, append, stream); return true;
         case 2: launch_decode<G, 2>(ka, n_kv, append, stream); return true;

@@ -152,6 +152,8 @@ def test_attention_after_append_uses_the_new_row(oracle, dev):
     (32, 8, 0, B.PATH_AUTO, 0), (32, 8, 15, B.PATH_SINGLE_PASS, 0), (32, 8, 16, B.PATH_SINGLE_PASS, 0),
     (32, 8, 1023, B.PATH_SPLIT_FUSED, 7), (32, 8, 1024, B.PATH_SPLIT_FUSED, 64), (64, 8, 777, B.PATH_AUTO, 0),
     (16, 8, 300, B.PATH_AUTO, 0), (12, 4, 333, B.PATH_SPLIT_FUSED, 5),
+    # groups of 8 query heads run 8 waves per workgroup, like the plain kernel (Qwen3-32B head layout)
+    (64, 8, 4096, B.PATH_AUTO, 0), (64, 8, 32768, B.PATH_AUTO, 0), (64, 8, 131072, B.PATH_AUTO, 0),
 ])
 def test_fused_append_attention(oracle, dev, layout, n_q, n_kv, ctx, path, splits):
     """llmi_hip_mha_decode_append (norm + rope + append + attention in one launch) against the oracle chain:
@@ -255,8 +257,7 @@ def _download(ptr, shape, dtype):
 def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout, layers, ctx):
     """Layers of (QK-Norm + RoPE + append, attention) at ctx + 1 new token: eager run and several replays
     of the captured graph all match the oracle layer by layer. 4 layers at ctx 300 in both layouts, and the
-    Qwen3-4B stack at its full size: 36 layers at ctx 4096 (the caches of the layers are one seeded cache
-    rotated by 37 positions per layer)."""
+    Qwen3-4B stack at its full size: 36 layers at ctx 4096, 36 independently seeded per-layer caches."""
     H = HostLib()
     n_q, n_kv, d = 32, 8, 128
     msl, pos, kv_dim = ctx + 1, ctx, n_kv * d
@@ -268,14 +269,9 @@ def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout, layers, 
         k_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
         v_all = np.zeros((layers, msl, kv_dim), dtype=np.uint16)
         raw = []
-        base = synth.make_case(400, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl) if layers > 4 else None
-        for l in range(layers):
-            if base is None:
-                c = synth.make_case(400 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
-                k_all[l], v_all[l] = c["k"][0], c["v"][0]
-            else:
-                k_all[l, :ctx] = np.roll(base["k"][0, :ctx], 37 * l, axis=0)
-                v_all[l, :ctx] = np.roll(base["v"][0, :ctx], 37 * l, axis=0)
+        for l in range(layers):  # every layer its own seeded cache
+            c = synth.make_case(400 + l, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+            k_all[l], v_all[l] = c["k"][0], c["v"][0]
             qr = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
             kr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
             vr = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))

@@ -59,6 +59,26 @@ def test_split_sweep_matches_oracle(oracle, dev, splits, waves, path):
     _check(oracle, dev, case, num_splits=splits, waves_per_group=waves, force_path=path)
 
 
+_LONG_REF = {}
+
+
+@pytest.mark.parametrize("splits", [4, 8, 16, 32, 64])
+@pytest.mark.parametrize("ctx", [8192, 16384, 32768])
+def test_split_sweep_long_context_matches_oracle(oracle, dev, ctx, splits):
+    """The long-context configuration at its full sizes: split counts 4 .. 64 at ctx 8192, 16384 and 32768
+    against the oracle (fused combine, 4 waves, head-major; the oracle runs once per context length)."""
+    case = synth.make_case(3, ctx=ctx, **QWEN3_4B)
+    if ctx not in _LONG_REF:
+        _LONG_REF[ctx] = run_oracle(oracle, case)
+    ref = _LONG_REF[ctx]
+    got16, got32, plan = run_hip(case, dev, want_plan=True, kv_layout=B.KV_LAYOUT_HEAD_MAJOR, force_path=B.PATH_SPLIT_FUSED,
+                                 num_splits=splits, waves_per_group=4)
+    assert plan.num_splits == splits and plan.path == B.PATH_SPLIT_FUSED
+    what = "ctx=%d splits=%d" % (ctx, splits)
+    assert_parity(got16, ref, "bf16 out " + what)
+    assert_tap_parity(got32, ref, what)
+
+
 @pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 159, 160, 161, 255, 256, 257, 1000, 4097])
 @pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT, B.PATH_SPLIT_FUSED])
 def test_ragged_lengths(oracle, dev, ctx, path):
