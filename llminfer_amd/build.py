@@ -27,14 +27,16 @@ def _run(cmd):
     return out
 
 
-def build_hip_library(verbose=False):
+def build_hip_library(verbose=False, defines=(), output=None):
+    """`defines`: extra NAME=VALUE macros (the kernels' build-time switches, e.g. LLMI_PV_VALU=1);
+    `output`: where to write a variant build instead of the in-tree library."""
     hipcc = os.environ.get("HIPCC", "hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
-    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES] + ["-o", LIB_PATH]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-D" + d for d in defines] + ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES] + ["-o", output or LIB_PATH]
     out = _run(cmd)
     if verbose and out.strip():
         print(out)
-    return LIB_PATH
+    return output or LIB_PATH
 
 
 def build_host_library(verbose=False):
@@ -62,6 +64,17 @@ def build_all(verbose=False):
 
 
 if __name__ == "__main__":
+    import argparse
+    ap = argparse.ArgumentParser(description="Builds the gfx950 library and the host layer in-tree, or a variant of the library.")
+    ap.add_argument("--define", action="append", default=[], metavar="NAME=VALUE",
+                    help="build-time switch of the kernels (LLMI_PV_VALU=1, LLMI_STAGES=3, ...); needs --output")
+    ap.add_argument("--output", default=None, help="write a variant of libllmi_hip.so here (load it with LLMI_HIP_LIBRARY)")
+    cli = ap.parse_args()
+    if cli.define or cli.output:
+        if not cli.output:
+            ap.error("--define needs --output: the in-tree library is always the default build")
+        print("built", build_hip_library(verbose=True, defines=cli.define, output=os.path.abspath(cli.output)))
+        sys.exit(0)
     for p in build_all(verbose=True):
         print("built", p)
     sys.exit(0)

@@ -84,6 +84,13 @@ constexpr int kCacheDevice = 16;
 #ifndef LLMI_MIN_WAVES_PER_EU
 #define LLMI_MIN_WAVES_PER_EU 2
 #endif
+#ifndef LLMI_PV_VALU
+// 1: the probability x value product runs on the vector ALU (fp32 multiply-adds with the
+// probabilities broadcast by DPP, the structure of the reference's inner loop,
+// code/source/op/kernel/cuda/mha_kernel.cu:114-155) instead of the matrix cores. Kept for the
+// side-by-side measurement that decides between the two; the library is built with 0.
+#define LLMI_PV_VALU 0
+#endif
 
 
 template <int I, int N, typename F>
@@ -344,6 +351,15 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     f32x4 o[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) o[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#if LLMI_PV_VALU
+    // Vector-ALU variant: ov[h][j] belongs to head h and column 8*n16 + j, summed over the rows
+    // 4*kg .. 4*kg+3 of every tile this wave has seen; the four DPP rows are added up after the loop.
+    float ov[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ov[h][j] = 0.0f;
+#endif
 
     // Each wave streams its tiles through a private ring of NSTAGE LDS slots
     // (8 KiB each: 4 KiB of K rows, 4 KiB of V rows) filled by LDS-DMA loads,
@@ -424,15 +440,42 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
         float p[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[i] = fast_exp2(s[i] - m_new);
+        const float psum = (p[0] + p[1]) + (p[2] + p[3]);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#if LLMI_PV_VALU
+        // Rescale only when some head's max moved (wave-uniform test); head h's factor sits in
+        // lane h of every 16-lane row.
+        if (__any(alpha != 1.0f)) {
+            static_for<0, G>([&](auto h) {
+                const float ah = row_bcast<h.value>(alpha);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ov[h.value][j] *= ah;
+            });
+        }
+        float vf[4][8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t w = r.v[i][j >> 1];
+                vf[i][j] = (j & 1) ? bf16_hi(w) : bf16_lo(w);
+            }
+        static_for<0, G>([&](auto h) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float ph = row_bcast<h.value>(p[i]);  // probability of (head h, row 4*kg + i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ov[h.value][j] = fmaf(ph, vf[i][j], ov[h.value][j]);
+            }
+        });
+#else
         // The probabilities enter the second MFMA as a sum of two bf16 numbers
         // (p = hi + lo, relative error 2^-17), so that the product keeps fp32-like accuracy.
         const uint32_t p01 = pack_bf16(p[0], p[1]);
         const uint32_t p23 = pack_bf16(p[2], p[3]);
         const uint32_t q01 = pack_bf16(p[0] - bf16_lo(p01), p[1] - bf16_hi(p01));
         const uint32_t q23 = pack_bf16(p[2] - bf16_lo(p23), p[3] - bf16_hi(p23));
-        const float psum = (p[0] + p[1]) + (p[2] + p[3]);
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
 
         // Rescale only when some head's max moved (wave-uniform test). The factor of
         // head 4*kg + r sits in lane 4*kg + r of this lane's 16-lane row.
@@ -462,6 +505,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
         for (int j = 0; j < 8; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb[j], o[j], 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pb, vb[j], o[j], 0, 0, 0);
+#endif
     };
 
     // Wave w owns tiles w, w+NW, ...: NSTAGE of them are always in flight.
@@ -571,6 +615,10 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
                     const uint32_t vw = vf[j >> 1];
                     const float vj = (j & 1) ? bf16_hi(vw) : bf16_lo(vw);
                     o[j] = f32x4{vj, vj, vj, vj};
+#if LLMI_PV_VALU
+#pragma unroll
+                    for (int h = 0; h < G; ++h) ov[h][j] = kg == 0 ? vj : 0.0f;
+#endif
                 }
             }
         }
@@ -590,6 +638,16 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     // The outputs are already summed over a wave's positions; the denominators are
     // per DPP row (kg) and share the running max of their head, so they add up plainly.
     l_run = rows_sum(l_run);
+#if LLMI_PV_VALU
+    // Into the layout the epilogue expects: o[j][r] of DPP row kg is head 4*kg + r.
+    static_for<0, G>([&](auto h) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float t = rows_sum(ov[h.value][j]);
+            if (kg == h.value / 4) o[j][h.value % 4] = t;
+        }
+    });
+#endif
 
     // This wave's ring is drained (every tile it issued was waited for and read).
     typedef float (*MergeS)[G];
