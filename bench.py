@@ -237,7 +237,7 @@ def stack_result(args, ctx):
             raise RuntimeError(host.llmi_host_last_error().decode())
 
     hidden = 2560 if n_q == 32 else 5120 if n_q == 64 else 1024
-    if args.stack_mode == 3:
+    if args.stack_mode in (3, 4):
         host.llmi_host_stack_enable_projections.argtypes = [ctypes.c_void_p, ctypes.c_int32]
         ok(host.llmi_host_stack_enable_projections(st, hidden))
     ok(host.llmi_host_stack_build_sincos(st))
@@ -255,7 +255,7 @@ def stack_result(args, ctx):
         up(host.llmi_host_stack_ptr(st, 4, l), synth.f32_to_bf16_bits(rng.standard_normal(KV_DIM).astype(np.float32)))
         up(host.llmi_host_stack_ptr(st, 5, l),
            synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * HEAD_DIM)).astype(np.float32)))
-    if args.stack_mode == 3:
+    if args.stack_mode in (3, 4):
         dim = n_q * HEAD_DIM
         for l in range(layers):
             up(host.llmi_host_stack_ptr(st, 12, l), synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32)))
@@ -280,7 +280,7 @@ def stack_result(args, ctx):
     ok(host.llmi_host_stack_replay(st, args.steps, ctypes.byref(ms)))
     us_token = ms.value * 1e3 / args.steps
     per_layer = algorithmic_bytes(pos + 1, n_q) + 23552  # + QK-Norm/RoPE/append traffic per layer
-    if args.stack_mode == 3:  # + both weight matrices, the hidden input and the residual (read + written)
+    if args.stack_mode in (3, 4):  # + both weight matrices, the hidden input and the residual (read + written)
         per_layer += ((n_q * HEAD_DIM + 2 * KV_DIM) * hidden + hidden * n_q * HEAD_DIM) * 2 + 3 * hidden * 2
     gbs = layers * per_layer / (us_token * 1e-6) / 1e9
     host.llmi_host_stack_destroy(st)
@@ -293,7 +293,9 @@ def stack_result(args, ctx):
                                % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major",
                                   "one launch per layer" if args.stack_mode == 2 else
                                   "three launches per layer: packed QKV GEMV (hidden %d), attention, output projection + "
-                                  "residual" % hidden if args.stack_mode == 3 else "two launches per layer")
+                                  "residual" % hidden if args.stack_mode == 3 else
+                                  "two launches per layer: packed QKV GEMV (hidden %d), attention whose idle workgroups do the "
+                                  "output projection + residual" % hidden if args.stack_mode == 4 else "two launches per layer")
                             + (", position read from device memory" if args.stack_follow_pos else "")},
         "us_per_layer": round(us_token / layers, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -519,7 +521,8 @@ def main():
     ap.add_argument("--stack-follow-pos", action="store_true",
                     help="with --stack: capture once for every position (kernels read it from device memory)")
     ap.add_argument("--stack-mode", type=int, default=2,
-                    help="with --stack: 3 = whole attention block (QKV GEMV, attention, o_proj + residual); "
+                    help="with --stack: 4 = whole attention block in two launches per layer (QKV GEMV, attention + o_proj + "
+                         "residual in one); 3 = the block in three launches (QKV GEMV, attention, o_proj + residual); "
                          "2 = norm/rope/append fused into the attention launch (default), "
                          "1 = separate kernel before attention (the reference's sequence)")
     args = ap.parse_args()

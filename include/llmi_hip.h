@@ -158,6 +158,26 @@ typedef struct llmi_mha_append_args {
  * The separate-combine path (LLMI_PATH_SPLIT) is not available here. */
 int llmi_hip_mha_decode_append(const llmi_mha_append_args* args);
 
+typedef struct llmi_attn_oproj_args {
+    llmi_mha_append_args attn; /* as for llmi_hip_mha_decode_append; attn.mha.output still receives the attention output */
+    const void* o_weight;      /* device bf16 [hidden][head_num*128] row-major: the layer's output projection         */
+    void* residual;            /* device bf16 [hidden]: residual += o_weight . attention output, rounded once          */
+    int32_t hidden;
+} llmi_attn_oproj_args;
+
+/* llmi_hip_mha_decode_append followed by llmi_hip_gemv in LLMI_GEMV_ADD_BF16 mode on its output: the tail of the
+ * reference's attention block, mha_kernel_cu then fused_gemv_add_kernel_cu (code/source/model/qwen3_fused.cpp:548-552;
+ * kernels mha_kernel.cu:440-529, matmul_kernel.cu:174-208) -- as ONE launch where the shape allows it. In that launch
+ * the workgroups that have handed their partial results over fetch the projection's weight rows while the combine
+ * still runs, wait (bounded, like the combine: llmi_hip_set_poll_limit, NaN on give-up) for the attention output and
+ * finish residual += W x. Same results as the two calls, bit for bit. The one-launch form needs: the fused split path
+ * with at least two splits and a host-side position, a query group of 1, 2, 4 or 8 heads, head_num*128 <= 4096,
+ * hidden <= 3 * (wavefronts of the workgroups that do not combine), a grid that fits the device's compute units at
+ * once, and head_num*4 more bytes of workspace than the plan reports. Anything else runs as the two launches.
+ * llmi_hip_mha_oproj_launches tells which: 1 or 2 (or a negative status for invalid arguments). */
+int llmi_hip_mha_decode_append_oproj(const llmi_attn_oproj_args* args);
+int llmi_hip_mha_oproj_launches(const llmi_attn_oproj_args* args);
+
 /* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len);
 

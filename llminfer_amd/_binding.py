@@ -42,6 +42,10 @@ class MhaAppendArgs(ctypes.Structure):
     ]
 
 
+class AttnOprojArgs(ctypes.Structure):
+    _fields_ = [("attn", MhaAppendArgs), ("o_weight", c_void_p), ("residual", c_void_p), ("hidden", c_i32)]
+
+
 class GemvArgs(ctypes.Structure):
     _fields_ = [
         ("input", c_void_p), ("weight", c_void_p), ("output", c_void_p),
@@ -97,6 +101,8 @@ SYMBOLS = {
     "llmi_hip_mha_decode": (ctypes.c_int, [ctypes.POINTER(MhaArgs)]),
     "llmi_hip_mha_decode_static": (ctypes.c_int, [ctypes.POINTER(MhaArgs)]),
     "llmi_hip_mha_decode_append": (ctypes.c_int, [ctypes.POINTER(MhaAppendArgs)]),
+    "llmi_hip_mha_decode_append_oproj": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
+    "llmi_hip_mha_oproj_launches": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
     "llmi_hip_mha_workspace_bytes": (c_size_t, [c_i32, c_i32, c_i32]),
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),
     "llmi_hip_sincos_table": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_void_p]),

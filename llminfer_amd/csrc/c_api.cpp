@@ -235,13 +235,76 @@ int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
     return launch_mha_decode(args->mha, plan, args);
 }
 
+// Validates the arguments and decides between the one-launch form (*fused = true, plan filled) and the pair.
+static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, bool* fused) {
+    if (!args) return LLMI_ERR_NULL_POINTER;
+    const llmi_mha_append_args& ap = args->attn;
+    if (!ap.key_new || !ap.value_new || !ap.norm_weight || !ap.sin_cache || !ap.cos_cache || !args->o_weight || !args->residual)
+        return LLMI_ERR_NULL_POINTER;
+    const void* ptrs[] = {ap.key_new, ap.value_new, ap.norm_weight, ap.sin_cache, ap.cos_cache, args->o_weight, args->residual};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
+    if (!(ap.eps >= 0.0f) || args->hidden <= 0) return LLMI_ERR_INVALID_ARG;
+    if (ap.mha.force_path == LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
+    if (int rc = make_plan(&ap.mha, plan, kMaxWaves, 1)) return rc;
+    *fused = false;
+    const llmi_mha_args& m = ap.mha;
+    const int n_kv = m.kv_dim / m.head_dim;
+    int32_t rows_per_wave = 0, max_k = 0;
+    oproj_limits(&rows_per_wave, &max_k);
+    const int64_t k = (int64_t)m.head_num * m.head_dim;
+    if (plan->path != LLMI_PATH_SPLIT_FUSED || plan->num_splits < 2 || m.pos_device) return LLMI_OK;
+    if (plan->group_pad > 8 || plan->waves_per_group != (plan->group_pad == 8 ? 8 : 4)) return LLMI_OK;
+    if (k % 512 != 0 || k > max_k) return LLMI_OK;
+    const int64_t worker_waves = (int64_t)n_kv * (plan->num_splits - 1) * plan->waves_per_group;
+    if (args->hidden > rows_per_wave * worker_waves) return LLMI_OK;
+    // every workgroup must be resident at once: the workers wait for the combiners
+    static std::atomic<int> cu_count{0};
+    int cus = cu_count.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return LLMI_OK;
+        }
+        cu_count.store(cus, std::memory_order_relaxed);
+    }
+    if ((int64_t)n_kv * plan->num_splits > cus) return LLMI_OK;
+    if (m.head_num > 128) return LLMI_OK;  // one wavefront collects the heads' tags, two per lane
+    if (m.workspace_bytes < plan->workspace_needed + (size_t)m.head_num * sizeof(uint32_t)) return LLMI_OK;
+    *fused = true;
+    return LLMI_OK;
+}
+
+int llmi_hip_mha_oproj_launches(const llmi_attn_oproj_args* args) {
+    llmi_mha_plan plan;
+    bool fused = false;
+    if (int rc = plan_oproj(args, &plan, &fused)) return rc;
+    return fused ? 1 : 2;
+}
+
+int llmi_hip_mha_decode_append_oproj(const llmi_attn_oproj_args* args) {
+    llmi_mha_plan plan;
+    bool fused = false;
+    if (int rc = plan_oproj(args, &plan, &fused)) return rc;
+    if (fused) return launch_mha_decode(args->attn.mha, plan, &args->attn, args);
+    if (int rc = launch_mha_decode(args->attn.mha, plan, &args->attn)) return rc;
+    const llmi_mha_args& m = args->attn.mha;
+    void* const out[3] = {args->residual, args->residual, args->residual};
+    const int32_t seg_end[3] = {args->hidden, args->hidden, args->hidden};
+    return launch_gemv(m.output, args->o_weight, out, seg_end, args->hidden, m.head_num * m.head_dim, LLMI_GEMV_ADD_BF16,
+                       static_cast<hipStream_t>(m.stream));
+}
+
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len) {
     if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     int splits = (max_seq_len + kTile - 1) / kTile;
     if (splits > kMaxSplits) splits = kMaxSplits;
     // Per head and split: head_dim partial outputs plus either (max, sum) as two floats
     // (separate combine kernel) or two 8-byte arrival records (fused combine).
-    return (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16;
+    // ... and, behind the records, one 4-byte counter per head for the fused output projection.
+    return (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16 +
+           (size_t)head_num * sizeof(uint32_t);
 }
 
 int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {

@@ -48,15 +48,6 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 
-__device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t ai = a[i], bi = b[i];  // (bit_cast straight from a vector element reads element 0)
-        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, ai), __builtin_bit_cast(bf16x2, bi), acc, false);
-    }
-    return acc;
-}
-
 struct GemvArgs {
     const uint16_t* x;   // [k]
     const uint16_t* w;   // [n][k]
@@ -90,12 +81,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_kernel(GemvArgs a) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) acc[r] = dot8(xv[u], wv[u][r], acc[r]);
+            for (int r = 0; r < kRows; ++r) acc[r] = dot8_bf16(xv[u], wv[u][r], acc[r]);
     }
     for (; c < a.k8; c += 64) {
         const u32x4 xv = x4[c];
 #pragma unroll
-        for (int r = 0; r < kRows; ++r) acc[r] = dot8(xv, __builtin_nontemporal_load(w4[r] + c), acc[r]);
+        for (int r = 0; r < kRows; ++r) acc[r] = dot8_bf16(xv, __builtin_nontemporal_load(w4[r] + c), acc[r]);
     }
 #pragma unroll
     for (int r = 0; r < kRows; ++r) acc[r] = wave_sum(acc[r]);

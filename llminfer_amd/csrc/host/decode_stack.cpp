@@ -82,7 +82,8 @@ void DecodeStack::build_sincos() {
 void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
     const bool with_qk_norm_rope = mode == kSeparateQkNormRope;
     LLMI_CHECK(!(follow_device_pos && with_qk_norm_rope));
-    const bool block = mode == kAttentionBlock;
+    const bool fused_tail = mode == kFusedBlock;  // the block with attention + output projection in one launch
+    const bool block = mode == kAttentionBlock || fused_tail;
     LLMI_CHECK(!block || hidden_dim_ > 0);
     const AttentionConfig& c = config_;
     tensor::Tensor& kc = buffers_->get_buffer(ModelBufferType::KeyCache);
@@ -161,12 +162,21 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
             f.sin_cache = buffers_->get_buffer(ModelBufferType::SinCache).ptr<float>();
             f.cos_cache = buffers_->get_buffer(ModelBufferType::CosCache).ptr<float>();
             f.eps = 1e-6f;
-            rc = llmi_hip_mha_decode_append(&f);
+            if (fused_tail) {
+                llmi_attn_oproj_args t{};
+                t.attn = f;
+                t.o_weight = out_weight(layer);
+                t.residual = residual();
+                t.hidden = hidden_dim_;
+                rc = llmi_hip_mha_decode_append_oproj(&t);
+            } else {
+                rc = llmi_hip_mha_decode_append(&f);
+            }
         } else {
             rc = llmi_hip_mha_decode(&m);
         }
         if (rc != LLMI_OK) LLMI_FATAL("decode attention: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
-        if (block) {
+        if (block && !fused_tail) {
             llmi_gemv_args o{};
             o.input = output(layer);
             o.weight = out_weight(layer);

@@ -54,7 +54,9 @@ public:
     // followed by attention (1, the reference's sequence), or both fused into one launch (2).
     // kAttentionBlock (3): packed QKV GEMV -> fused append attention -> output projection + residual,
     // three launches per layer.
-    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2, kAttentionBlock = 3 };
+    // kFusedBlock (4): the same block in two launches per layer: packed QKV GEMV -> attention whose idle
+    // workgroups also do the output projection + residual (llmi_hip_mha_decode_append_oproj).
+    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2, kAttentionBlock = 3, kFusedBlock = 4 };
     // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
     // `follow_device_pos`: the kernels read the position from the stack's device word (set_position)
     // and `pos` is the largest position they may see; modes 0 and 2 only (the separate QK-Norm/RoPE

@@ -35,7 +35,11 @@ int read_poll_timeouts(unsigned long long* count);
 int poll_limit();
 
 // `append` non-null: the fused QK-Norm + RoPE + K/V append variant.
-int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append = nullptr);
+// `oproj` non-null (with `append`): the attention launch also computes the output projection + residual add.
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append = nullptr,
+                      const llmi_attn_oproj_args* oproj = nullptr);
+// What the fused projection holds per wavefront: weight rows, and the widest attention output (elements).
+int oproj_limits(int32_t* rows_per_wave, int32_t* max_k);
 int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);
 int launch_sincos_table(float* sin_cache, float* cos_cache, int32_t head_dim, int32_t max_seq_len,
                         hipStream_t stream);

@@ -74,6 +74,10 @@ __device__ unsigned int g_poll_timeouts = 0;
 
 constexpr int kTile = 16;      // positions per MFMA tile
 constexpr int kHeadDim = 128;
+// Fused output projection: weight rows a wavefront holds in registers while it waits for the attention
+// output, and 512-element steps per row (kOprojSteps * 512 = the widest attention output it takes).
+constexpr int kOprojRows = 3;
+constexpr int kOprojSteps = 8;
 // Cache policy of the buffer loads and stores that hand partial results from one workgroup to
 // another: the instruction's sc1 bit, device scope (served by memory, coherent across the XCDs).
 constexpr int kCacheDevice = 16;
@@ -83,6 +87,11 @@ constexpr int kCacheDevice = 16;
 #endif
 #ifndef LLMI_MIN_WAVES_PER_EU
 #define LLMI_MIN_WAVES_PER_EU 2
+#endif
+#ifndef LLMI_OPROJ_PREFETCH_ROWS
+// Weight rows (of 3 per wavefront) the fused output projection requests before it waits for the
+// attention output; the others are requested after the wait.
+#define LLMI_OPROJ_PREFETCH_ROWS 3
 #endif
 #ifndef LLMI_PV_VALU
 // 1: the probability x value product runs on the vector ALU (fp32 multiply-adds with the
@@ -231,6 +240,18 @@ struct KernelArgs {
     const float* cos_cache;
     int64_t slot_head_stride;  // elements between KV heads inside a slot
     float eps;
+    // Fused output projection (OPROJ kernels only): after the attention the workgroups that do not
+    // combine compute residual[r] += o_w[r] . out for their share of the rows.
+    uint32_t* ready;         // in the workspace: [0] generation word, [4 + hq] "head hq's output is written" = generation + 1
+    const uint16_t* o_w;     // [o_n][n_q * 128] bf16, row-major
+    uint16_t* o_res;         // [o_n] bf16 residual stream, updated in place
+    int32_t o_n;             // rows (the model's hidden size)
+};
+
+// What the attention part of an OPROJ kernel hands to the projection part.
+struct OprojState {
+    uint32_t gen_base = 0u;  // the generation word as read before this workgroup published anything
+    bool worker = false;     // this workgroup takes rows of the projection (it is not a combiner)
 };
 
 // RMSNorm * weight + half-rotation RoPE of 128-wide bf16 rows held in LDS, in place, by one
@@ -286,8 +307,8 @@ __device__ __forceinline__ void norm_rope_rows_lds(char* rows, const char* w, co
 template <int G, int NW>
 constexpr int kWavesPerEu = (G >= 16 && NW != 2) ? 1 : LLMI_MIN_WAVES_PER_EU;
 
-template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
-__global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kernel(KernelArgs a) {
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER, bool OPROJ>
+__device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState& proj) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
@@ -529,6 +550,14 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     // and the first tile is worked on as soon as it lands. As ordinary loads their wait would be
     // placed by the compiler, which does not know about the DMA loads: it would also wait for
     // every tile issued before that point.
+    if constexpr (OPROJ) {
+        // The generation word moves once per launch, after every head's output is written. That needs
+        // every combiner, each combiner needs the records of its splits, and those go out only after
+        // every load of this wavefront has come back (the wait in front of the record stores): read
+        // here, the word still holds the value of before, in every workgroup of the grid. Issued ahead of
+        // the tiles, so that nothing near the end of the kernel has to wait for it.
+        proj.gen_base = __hip_atomic_load(a.ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     char* shared_staging = smem + kStagingBase;                                     // append variant only
     char* my_rows = smem + kStagingBase + (kSharedSlots + wave * kQSlots) * 1024;  // this wave's query rows
     {
@@ -671,6 +700,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     __syncthreads();
 
     const bool fused = a.records != nullptr && n_active > 1;
+    if constexpr (OPROJ) proj.worker = split != n_active - 1;
     // One thread per (head, 16-byte column): weights e^(m_w - M) of the waves, weighted sum.
     const int n_units = a.group * (kHeadDim / 4);
     const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -895,11 +925,40 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
                 // A wait that ran out of patience poisons the output rather than returning a partial sum.
                 const float inv = arrived ? 1.0f / den : __builtin_nanf("");
                 const f32x4 r = acc * inv;
-                *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
+                const unsigned long long packed = (unsigned long long)pack_bf16(r[0], r[1]) | ((unsigned long long)pack_bf16(r[2], r[3]) << 32);
+                unsigned long long* op = reinterpret_cast<unsigned long long*>(a.out + (int64_t)hq * kHeadDim + c4 * 4);
+                if constexpr (OPROJ) __hip_atomic_store(op, packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // read by other workgroups in this launch
+                else *op = packed;
                 if (a.out_f32) {
                     float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
 #pragma unroll
                     for (int e = 0; e < 4; ++e) of[e] = r[e];
+                }
+            }
+            if constexpr (OPROJ) {
+                // The head's output is acknowledged: say so, with the generation this launch will end on.
+                // (Every workgroup of the grid read the same generation word: it moves only after all
+                // heads are done.) The workers wait for all heads' tags; one wavefront of the grid (head 0
+                // of the last KV head, whose workgroup is dispatched last) does too and then moves the
+                // word for the next launch -- also when its wait gives up, so that tags left behind by
+                // this launch can never match the next one.
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                uint32_t* done = a.ready + 4;
+                const uint32_t target = proj.gen_base + 1u;
+                if (lane == 0) __hip_atomic_store(done + hq, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (kvh == (int)gridDim.x - 1 && h == 0) {
+                    bool all_done = false;
+                    for (int spin = 0; spin < a.max_polls; ++spin) {
+                        const uint32_t d0 = __hip_atomic_load(done + min(lane, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        const uint32_t d1 = __hip_atomic_load(done + min(lane + 64, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        all_done = __all(d0 == target && d1 == target);
+                        if (all_done) break;
+                        __builtin_amdgcn_s_sleep(8);
+                    }
+                    if (lane == 0) {
+                        __hip_atomic_store(a.ready, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (!all_done) atomicAdd(&g_poll_timeouts, 1u);
+                    }
                 }
             }
         };
@@ -987,6 +1046,104 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
     }
 }
 
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
+__global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kernel(KernelArgs a) {
+    OprojState unused;
+    mha_decode_body<G, NW, NSTAGE, APPEND, DYN, STAGGER, false>(a, unused);
+}
+
+// The attention launch with the layer's output projection and residual add behind it, in the same launch
+// (role of the pair mha_kernel_cu + fused_gemv_add_kernel_cu, code/source/model/qwen3_fused.cpp:548-552).
+// A workgroup that has handed its partial results over (every one but the combiners) is idle while the
+// combine runs: it requests its share of the projection's weight rows -- they do not depend on the
+// attention -- and holds them in registers, waits (bounded) for every head's tag of this launch, reads the
+// attention output with device-coherent loads and finishes its rows: dot products, residual add, one
+// rounding. The weights stream while HBM would otherwise sit idle behind the attention's hand-over.
+// Needs every workgroup of the grid resident at once (the launcher checks the grid against the CU count).
+template <int G, int NW, int NSTAGE>
+__global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_oproj_kernel(KernelArgs a) {
+    OprojState proj;
+    mha_decode_body<G, NW, NSTAGE, true, false, false, true>(a, proj);
+    if (!proj.worker) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_kv = gridDim.x;
+    // Rows are dealt to the wavefronts of the workers in turn: wavefront w takes rows w, w + W, w + 2W.
+    const int n_waves = n_kv * ((int)gridDim.y - 1) * NW;
+    const int gw = ((int)blockIdx.y * n_kv + (int)blockIdx.x) * NW + wave;
+    constexpr int kRows = kOprojRows, kSteps = kOprojSteps;
+    const int k16 = a.n_q * (kHeadDim / 8);  // 16-byte chunks per weight row
+    const int steps = k16 >> 6;
+    const u32x4* w4 = reinterpret_cast<const u32x4*>(a.o_w);
+    u32x4 wv[kRows][kSteps];
+    int row[kRows];
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+        row[i] = gw + i * n_waves;
+        const u32x4* wr = w4 + (int64_t)min(row[i], a.o_n - 1) * k16 + lane;  // rows past the end repeat the last one and are not written
+        if (i < LLMI_OPROJ_PREFETCH_ROWS) {
+#pragma unroll
+            for (int t = 0; t < kSteps; ++t)
+                if (t < steps) wv[i][t] = __builtin_nontemporal_load(wr + t * 64);
+        }
+    }
+    // (the residual values these rows are added to travel with the weights)
+    float res_in[kRows];
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) res_in[i] = bf16_lo((uint32_t)a.o_res[min(row[i], a.o_n - 1)]);
+    // Bounded wait for the attention output: every head carries this launch's tag. One wavefront per
+    // workgroup polls (a thousand wavefronts polling one line slow everything that shares its channel).
+    __shared__ int s_seen;
+    if (wave == 0) {
+        const uint32_t* done = a.ready + 4;
+        const uint32_t target = proj.gen_base + 1u;
+        bool seen = false;
+        for (int spin = 0; spin < a.max_polls; ++spin) {
+            const uint32_t d0 = __hip_atomic_load(done + min(lane, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t d1 = __hip_atomic_load(done + min(lane + 64, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            seen = __all(d0 == target && d1 == target);
+            if (seen) break;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (lane == 0) {
+            s_seen = seen ? 1 : 0;
+            if (!seen) atomicAdd(&g_poll_timeouts, 1u);
+        }
+    }
+    __syncthreads();
+    const bool ok = s_seen != 0;
+    // (rows beyond the prefetch depth are fetched now)
+#pragma unroll
+    for (int i = LLMI_OPROJ_PREFETCH_ROWS; i < kRows; ++i) {
+        const u32x4* wr = w4 + (int64_t)min(row[i], a.o_n - 1) * k16 + lane;
+#pragma unroll
+        for (int t = 0; t < kSteps; ++t)
+            if (t < steps) wv[i][t] = __builtin_nontemporal_load(wr + t * 64);
+    }
+    // The attention output was written through to memory before the word moved, and no cache on this
+    // side can hold an older copy: nothing in this launch has read it before, and caches do not keep
+    // lines across launches. Ordinary loads, so that an XCD's L2 fetches the 8 KiB once for all its
+    // workgroups (a thousand device-coherent reads of the same lines would queue at one memory channel).
+    const u32x4* x4 = reinterpret_cast<const u32x4*>(a.out);
+    u32x4 xv[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t)
+        if (t < steps) xv[t] = x4[t * 64 + lane];
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int t = 0; t < kSteps; ++t)
+            if (t < steps) acc = dot8_bf16(xv[t], wv[i][t], acc);
+        acc = wave_sum(acc);
+        if (lane == 0 && row[i] < a.o_n) {
+            // fp32 + fp32 -> bf16 once, like fused_gemv_add (matmul_kernel.cu:169-170); a wait that gave up poisons the row
+            const float sum = ok ? acc + res_in[i] : __builtin_nanf("");
+            a.o_res[row[i]] = f32_to_bf16(sum);
+        }
+    }
+}
+
 // Log-sum-exp merge of the split partials of one query head
 // (role of flashdecoding_gqa_combine_kernel, mha_kernel.cu:399-438).
 __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __restrict__ ws,
@@ -1066,7 +1223,19 @@ bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipSt
     }
 }
 
+template <int G, int NW>
+void launch_oproj(const KernelArgs& ka, int n_kv, hipStream_t stream) {
+    constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
+    hipLaunchKernelGGL((mha_oproj_kernel<G, NW, kStages>), dim3(n_kv, ka.num_splits), dim3(NW * 64), 0, stream, ka);
+}
+
 }  // namespace
+
+int oproj_limits(int32_t* rows_per_wave, int32_t* max_k) {
+    *rows_per_wave = kOprojRows;
+    *max_k = kOprojSteps * 512;
+    return LLMI_OK;
+}
 
 int static_scratch(void** ptr, size_t* bytes) {
     // One address per device, looked up with that device current the first time it is asked for.
@@ -1096,7 +1265,8 @@ int read_poll_timeouts(unsigned long long* count) {
     return LLMI_OK;
 }
 
-int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append) {
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append,
+                      const llmi_attn_oproj_args* oproj) {
     const int n_kv = args.kv_dim / args.head_dim;
     const int64_t layer_off = (int64_t)args.layer_id * args.max_seq_len * args.kv_dim;
 
@@ -1146,10 +1316,26 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         ka.slot_head_stride = ka.head_stride;
         ka.eps = append->eps;
     }
+    if (oproj) {
+        // The generation word and the per-head tags sit behind the arrival records (the caller has checked that they fit).
+        ka.ready = reinterpret_cast<uint32_t*>(ka.records + (size_t)args.head_num * plan.num_splits * 2);
+        ka.o_w = static_cast<const uint16_t*>(oproj->o_weight);
+        ka.o_res = static_cast<uint16_t*>(oproj->residual);
+        ka.o_n = oproj->hidden;
+    }
 
     hipStream_t stream = static_cast<hipStream_t>(args.stream);
     const bool ap = append != nullptr;
     bool ok = false;
+    if (oproj) {
+        // (the caller has checked the shape: fused split path, 4 waves, or 8 for groups of 8 heads)
+        if (plan.group_pad == 1 && plan.waves_per_group == 4) launch_oproj<1, 4>(ka, n_kv, stream), ok = true;
+        else if (plan.group_pad == 2 && plan.waves_per_group == 4) launch_oproj<2, 4>(ka, n_kv, stream), ok = true;
+        else if (plan.group_pad == 4 && plan.waves_per_group == 4) launch_oproj<4, 4>(ka, n_kv, stream), ok = true;
+        else if (plan.group_pad == 8 && plan.waves_per_group == 8) launch_oproj<8, 8>(ka, n_kv, stream), ok = true;
+        if (!ok) return LLMI_ERR_INVALID_ARG;
+        return check_launch();
+    }
     switch (plan.group_pad) {
         case 1: ok = launch_decode_nw<1>(ka, n_kv, plan.waves_per_group, ap, stream); break;
         case 2: ok = launch_decode_nw<2>(ka, n_kv, plan.waves_per_group, ap, stream); break;

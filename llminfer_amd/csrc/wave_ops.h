@@ -35,6 +35,18 @@ __device__ __forceinline__ float wave_sum(float x) {
     return (row_lane0(x, 0) + row_lane0(x, 1)) + (row_lane0(x, 2) + row_lane0(x, 3));
 }
 
+// acc + the dot product of eight bf16 pairs (two 16-byte operands), fp32 accumulate, left to right.
+typedef uint32_t wave_ops_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float dot8_bf16(wave_ops_u32x4 a, wave_ops_u32x4 b, float acc) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t ai = a[i], bi = b[i];  // (bit_cast straight from a vector element reads element 0)
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, ai), __builtin_bit_cast(bf16x2, bi), acc, false);
+    }
+    return acc;
+}
+
 }  // namespace llmi
 
 #endif

@@ -106,8 +106,9 @@ def qk_norm_rope_append(query, key_new, value_new, key_cache, value_cache, norm_
 
 
 def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos_cache, key_cache, value_cache,
-                      output, workspace, *, eps=1e-6, stream=None, **kw):
-    """QK-Norm + RoPE + K/V append + decode attention as one kernel (llmi_hip_mha_decode_append)."""
+                      output, workspace, *, eps=1e-6, stream=None, o_weight=None, residual=None, **kw):
+    """QK-Norm + RoPE + K/V append + decode attention as one kernel (llmi_hip_mha_decode_append). With `o_weight`
+    [hidden][head_num*128] and `residual` [hidden]: llmi_hip_mha_decode_append_oproj; returns the launch count."""
     for name, t in (("query_raw", query_raw), ("key_new", key_new), ("value_new", value_new),
                     ("norm_weight", norm_weight), ("key_cache", key_cache), ("value_cache", value_cache),
                     ("output", output)):
@@ -119,8 +120,17 @@ def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos
     a.mha = make_mha_args(query_raw, key_cache, value_cache, output, workspace, stream=_stream_handle(stream), **kw)
     a.key_new, a.value_new, a.norm_weight = _ptr(key_new), _ptr(value_new), _ptr(norm_weight)
     a.sin_cache, a.cos_cache, a.eps = _ptr(sin_cache), _ptr(cos_cache), eps
-    B.check(B.lib().llmi_hip_mha_decode_append(ctypes.byref(a)), "llmi_hip_mha_decode_append")
-    return output
+    if o_weight is None:
+        B.check(B.lib().llmi_hip_mha_decode_append(ctypes.byref(a)), "llmi_hip_mha_decode_append")
+        return output
+    # ... with the layer's output projection and residual add behind it (llmi_hip_mha_decode_append_oproj)
+    _check_dev("o_weight", o_weight, _BF16_DTYPES)
+    _check_dev("residual", residual, _BF16_DTYPES)
+    t = B.AttnOprojArgs()
+    t.attn, t.o_weight, t.residual, t.hidden = a, _ptr(o_weight), _ptr(residual), residual.numel()
+    launches = B.lib().llmi_hip_mha_oproj_launches(ctypes.byref(t))
+    B.check(B.lib().llmi_hip_mha_decode_append_oproj(ctypes.byref(t)), "llmi_hip_mha_decode_append_oproj")
+    return launches
 
 
 def sincos_table(head_dim, max_seq_len, device="cuda", stream=None):

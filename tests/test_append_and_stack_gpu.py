@@ -372,10 +372,12 @@ def test_decode_stack_graph_follows_the_device_position(oracle, dev):
         H.L.llmi_host_stack_destroy(stack)
 
 
-def test_attention_block_stack_matches_the_oracle_chain(oracle, dev):
-    """Mode 3 of the stack, two layers: packed QKV GEMV -> QK-Norm + RoPE + append + attention -> output
-    projection added to the residual stream. The oracle replays the chain with a bf16 rounding wherever
-    the kernels store bf16 (GEMV outputs, attention output, residual)."""
+@pytest.mark.parametrize("mode", [3, 4])
+def test_attention_block_stack_matches_the_oracle_chain(oracle, dev, mode):
+    """Modes 3 and 4 of the stack, two layers: packed QKV GEMV -> QK-Norm + RoPE + append + attention -> output
+    projection added to the residual stream (mode 4: attention and projection in one launch). The oracle
+    replays the chain with a bf16 rounding wherever the kernels store bf16 (GEMV outputs, attention
+    output, residual)."""
     H = HostLib()
     H.L.llmi_host_stack_enable_projections.argtypes = [ctypes.c_void_p, ctypes.c_int32]
     layers, ctx, n_q, n_kv, d, hidden, layout = 2, 280, 16, 8, 128, 1024, B.KV_LAYOUT_HEAD_MAJOR
@@ -416,7 +418,7 @@ def test_attention_block_stack_matches_the_oracle_chain(oracle, dev):
         _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), synth.to_head_major(k_up, n_kv))
         _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), synth.to_head_major(v_up, n_kv))
         _upload(H.L.llmi_host_stack_ptr(stack, 13, 0), res0)
-        H.ok(H.L.llmi_host_stack_run(stack, pos, 3))
+        H.ok(H.L.llmi_host_stack_run(stack, pos, mode))
         for l in range(layers):
             got = _download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16)
             assert_parity(synth.bf16_bits_to_f32(got), attn_refs[l], "block layer %d attention" % l)
@@ -425,13 +427,74 @@ def test_attention_block_stack_matches_the_oracle_chain(oracle, dev):
         assert np.all(np.abs(res - res_ref) <= np.abs(res_ref) / 64 + 2e-2), np.abs(res - res_ref).max()
         # graph replay of the block gives the same residual increment again
         _upload(H.L.llmi_host_stack_ptr(stack, 13, 0), res0)
-        H.ok(H.L.llmi_host_stack_capture(stack, pos, 3))
+        H.ok(H.L.llmi_host_stack_capture(stack, pos, mode))
         ms = ctypes.c_float()
-        H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
-        res2 = synth.bf16_bits_to_f32(_download(H.L.llmi_host_stack_ptr(stack, 13, 0), (hidden,), np.uint16))
-        assert np.array_equal(res, res2)
+        for rep in range(3):  # replays of one graph: the per-head counters of the fused projection keep moving
+            _upload(H.L.llmi_host_stack_ptr(stack, 13, 0), res0)
+            H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
+            res2 = synth.bf16_bits_to_f32(_download(H.L.llmi_host_stack_ptr(stack, 13, 0), (hidden,), np.uint16))
+            assert np.array_equal(res, res2), "replay %d" % rep
+            torch.randn(1000, device=dev).sum().item()  # eager work between replays
     finally:
         H.L.llmi_host_stack_destroy(stack)
+
+
+@pytest.mark.parametrize("n_q,ctx,hidden,want_launches,extra", [
+    (32, 4096, 2560, 1, {}),      # Qwen3-4B: 32 splits, 248 worker workgroups, rows dealt 3 / 3 / 2 per wavefront
+    (32, 1500, 2560, 1, {}),
+    (16, 700, 1024, 1, {}),       # Qwen3-0.6B head layout
+    (64, 5000, 640, 2, {}),       # attention output wider than the fused form takes: two launches, same answer
+    (32, 100, 2560, 2, {}),       # single pass: nothing idles, two launches
+    (32, 4096, 2560, 2, {"num_splits": 2, "force_path": B.PATH_SPLIT_FUSED}),  # too few workers for 2560 rows
+])
+def test_fused_output_projection_equals_attention_then_gemv_add(oracle, dev, n_q, ctx, hidden, want_launches, extra):
+    """llmi_hip_mha_decode_append_oproj against llmi_hip_mha_decode_append followed by llmi_hip_gemv (add mode) on
+    the same inputs: same attention output and same residual bit for bit, whichever form runs; the attention
+    output also against the oracle. Called three times in a row on one workspace (its per-head counters move on)."""
+    n_kv, d = 8, 128
+    rng = np.random.RandomState(ctx + hidden)
+    msl, pos, kv_dim, dim = ctx + 2, ctx, n_kv * d, n_q * d
+    case = synth.make_case(900 + ctx, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+    k0, v0 = case["k"].copy(), case["v"].copy()
+    q_raw = synth.f32_to_bf16_bits(rng.standard_normal((n_q, d)).astype(np.float32))
+    k_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    v_new = synth.f32_to_bf16_bits(rng.standard_normal((n_kv, d)).astype(np.float32))
+    w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+    wo = synth.f32_to_bf16_bits((rng.standard_normal((hidden, dim)) / np.sqrt(dim)).astype(np.float32))
+    res0 = synth.f32_to_bf16_bits(rng.standard_normal(hidden).astype(np.float32))
+    sin_o, cos_o = oracle.sincos_table(d, msl)
+    k_ref, v_ref = k0.copy(), v0.copy()
+    k_ref[0, pos] = oracle.qk_norm_rope(k_new, w[d:], sin_o[pos], cos_o[pos]).reshape(-1)
+    v_ref[0, pos] = v_new.reshape(-1)
+    q_n = oracle.qk_norm_rope(q_raw, w[:d], sin_o[pos], cos_o[pos])
+    ref = oracle.mha_cpu(q_n.reshape(-1), k_ref, v_ref, 0, pos, kv_dim, n_q // n_kv, n_q, d, msl)
+
+    sin_d, cos_d = ops.sincos_table(d, msl, dev)
+    wo_d, w_d = to_dev(wo.reshape(-1), dev), to_dev(w, dev)
+    qd, kd, vd = to_dev(q_raw.reshape(-1), dev), to_dev(k_new.reshape(-1), dev), to_dev(v_new.reshape(-1), dev)
+    ws = torch.full((ops.workspace_bytes(n_q, d, msl) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    kw = dict(layer_id=0, pos=pos, kv_dim=kv_dim, kv_mul=n_q // n_kv, head_num=n_q, head_dim=d, max_seq_len=msl,
+              kv_layout=B.KV_LAYOUT_HEAD_MAJOR, **extra)
+
+    def fresh():
+        return (to_dev(synth.to_head_major(k0, n_kv), dev), to_dev(synth.to_head_major(v0, n_kv), dev),
+                torch.zeros(dim, dtype=torch.int16, device=dev), to_dev(res0, dev))
+
+    # the two-call form
+    kc, vc, out_a, res_a = fresh()
+    ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_a, ws, **kw)
+    ops.gemv(out_a, wo_d.view(hidden, dim), res_a, mode=B.GEMV_ADD_BF16)
+    torch.cuda.synchronize()
+    assert_parity(from_dev_bf16(out_a), ref, "attention in front of the projection")
+    for call in range(3):
+        kc, vc, out_b, res_b = fresh()
+        launches = ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_b, ws, o_weight=wo_d, residual=res_b, **kw)
+        torch.cuda.synchronize()
+        assert launches == want_launches
+        assert torch.equal(out_b, out_a), "call %d: attention outputs differ" % call
+        assert torch.equal(res_b, res_a), "call %d: residuals differ" % call
+    n = ctypes.c_uint64()
+    assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(n)) == 0
 
 
 def test_mha_op_forward_through_registry_hook(oracle, dev):
