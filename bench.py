@@ -423,8 +423,7 @@ def dispatch_rows(sw, ctx_list):
     for ctx in ctx_list:
         def timed(**over):
             return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over))
-        if not rows:
-            timed()  # the first graph timed in a process runs 1-2 us per call slow: discard one
+        timed()  # the first graph timed on a context's slices runs up to a microsecond per call slow: discard one
         auto = timed()
         alts = {}
         if ctx <= 1024:
@@ -433,6 +432,7 @@ def dispatch_rows(sw, ctx_list):
         for sp in (4, 8, 16, 32, 64):
             if sp <= tiles:
                 alts["split%d" % sp] = timed(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
+        auto = min(auto, timed())  # (and once more at the end: the automatic plan is one of the forced ones)
         best = min(alts, key=alts.get)
         p = sw.plan(ctx)
         rows.append({"ctx": ctx, "auto_us": round(auto, 2), "auto_plan": "path%d S=%d W=%d" % (p.path, p.num_splits, p.waves_per_group),
@@ -591,8 +591,15 @@ def main():
         return seq
 
     timed_seq = replays_for(args.steps)  # (captured before the clock starts)
-    if args.warmup:
-        sw.time_replays(replays_for(args.warmup))
+    warm_seq = replays_for(args.warmup) if args.warmup else []
+    # Set-up, like the arena fill: a fifth of a second of the same work lets the clocks settle (a cold device
+    # runs the first milliseconds 5-8 % slow), so that short --steps / --warmup values measure the steady state
+    # too. These replays are neither warm-up steps nor timed.
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < 0.2:
+        sw.time_replays([(g_full, 20)])
+    if warm_seq:
+        sw.time_replays(warm_seq)
     ms = sw.time_replays(timed_seq)
     steps = args.steps
     ms_per_step = ms / steps

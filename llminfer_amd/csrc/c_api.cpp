@@ -108,7 +108,10 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
     const size_t per_split_fused = (size_t)a->head_num * (a->head_dim * sizeof(float) + 2 * sizeof(unsigned long long));
 
     const int single_waves_max = (max_waves < wave_cap ? max_waves : wave_cap);  // 8 where the kernel variant allows
-    const int single_pass_max = kSinglePassMaxLen;
+    // Groups of 8 query heads run 8 waves per workgroup, which carry a single pass a little further
+    // (64 query / 8 KV heads: single pass 4.96 / 5.36 us against 5.47 / 5.61 us split at 176 / 208
+    // positions, 6.30 against 5.71 at 256).
+    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 208 : kSinglePassMaxLen;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
@@ -143,7 +146,11 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             if (half < 2) half = 2;
             int quarter = half / 2;
             if (quarter < 2) quarter = 2;
-            want = tiles >= target ? target : tiles >= half ? half : quarter;
+            // With 8 waves per workgroup a split wants four tiles before one workgroup per CU pays
+            // (64 query / 8 KV heads, 16 against 32 splits: 6.13 : 6.94 us at 512 positions, 6.65 : 7.12
+            // at 1024, 7.22 : 7.70 at 1500; 32 splits ahead from 2048).
+            const int full = target * (waves == 8 ? 4 : 1);
+            want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;
             const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
