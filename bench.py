@@ -27,7 +27,15 @@ N_Q, N_KV, HEAD_DIM = 32, 8, 128
 KV_DIM = N_KV * HEAD_DIM
 HBM_PEAK_GBS = 8000.0
 DEFAULT_CTX = [1024, 2048, 4096, 8192, 16384, 32768]
-SLICES = 8  # distinct KV slices per context length inside one captured graph
+SLICES = 8  # steps (one KV slice per context each) inside one captured graph of the sweep
+SLICE_SET_BYTES = 512 << 20  # a context's slices together are at least this big: twice the 256 MB Infinity Cache
+
+
+def n_slices(ctx):
+    """Distinct KV slices of one context length: at least SLICES, and enough that replaying one length alone
+    still walks more K/V bytes than the Infinity Cache holds before a slice comes round again."""
+    per_slice = 2 * ctx * KV_DIM * 2
+    return min(128, max(SLICES, -(-SLICE_SET_BYTES // per_slice)))  # (128 slices at most: below 1024 positions a call is all latency)
 
 
 def algorithmic_bytes(ctx, n_q=N_Q, n_kv=N_KV):
@@ -38,7 +46,7 @@ def algorithmic_bytes(ctx, n_q=N_Q, n_kv=N_KV):
 def make_arena(torch, dev, ctx_list, n_q=N_Q):
     """One K and one V slab; each (ctx, slice) pair owns a distinct region. Values: N(0,1),
     RMS-normalised per 128-wide head vector, rounded to bf16."""
-    total_rows = sum(ctx_list) * SLICES
+    total_rows = sum(c * n_slices(c) for c in ctx_list)
     gen = torch.Generator(device=dev)
     gen.manual_seed(20260614)
 
@@ -55,7 +63,7 @@ def make_arena(torch, dev, ctx_list, n_q=N_Q):
     regions = {}
     row = 0
     for ctx in ctx_list:
-        for s in range(SLICES):
+        for s in range(n_slices(ctx)):
             regions[(ctx, s)] = row * KV_DIM  # element offset of a [N_KV][ctx][128] cache
             row += ctx
     q = torch.randn((n_q, HEAD_DIM), generator=gen, device=dev)
@@ -338,10 +346,10 @@ class Sweep:
         return self.ops.mha_plan(self.call_args(ctx, 0, **over))
 
     def enqueue(self, ctxs, first_step, steps, **over):
-        """Steps first_step .. first_step+steps-1: one call per context each, on slice step % SLICES."""
+        """Steps first_step .. first_step+steps-1: one call per context each, on slice step % n_slices(ctx)."""
         for s in range(first_step, first_step + steps):
             for ctx in ctxs:
-                a = self.call_args(ctx, s % SLICES, **over)
+                a = self.call_args(ctx, s % n_slices(ctx), **over)
                 a.stream = self.stream.cuda_stream
                 self.B.check(self.decode(ctypes.byref(a)), "llmi_hip_mha_decode")
 
@@ -349,7 +357,7 @@ class Sweep:
         probe = self.B.lib().llmi_hip_probe_stream_read
         for s in range(first_step, first_step + steps):
             for ctx in ctxs:
-                off = self.regions[(ctx, s % SLICES)] * 2
+                off = self.regions[(ctx, s % n_slices(ctx))] * 2
                 self.B.check(probe(self.k.data_ptr() + off, self.v.data_ptr() + off, ctx * KV_DIM * 2, workgroups, waves,
                                    inflight, self.sink.data_ptr(), self.stream.cuda_stream), "llmi_hip_probe_stream_read")
 
@@ -379,13 +387,14 @@ class Sweep:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1)
 
-    def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None):
-        """Best of `reps` batches of graph replays, us per call."""
-        g = self.capture(enqueue_fn)
-        self.time_replays([(g, 8)])
-        n = replays or 40
+    def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None, steps=SLICES):
+        """Best of `reps` batches of graph replays (a graph of `steps` steps), us per call."""
+        g = self.capture(enqueue_fn, steps)
+        scale = max(1, steps // SLICES)
+        self.time_replays([(g, max(1, 8 // scale))])
+        n = max(1, (replays or 40) // scale)
         best = min(self.time_replays([(g, n)]) for _ in range(reps))
-        return best * 1e3 / (n * SLICES * calls_per_step)
+        return best * 1e3 / (n * steps * calls_per_step)
 
 
 # stream-only configurations tried for the floor: (workgroups, waves per workgroup, tiles in flight per wave)
@@ -402,7 +411,7 @@ def stream_floor(sw, ctx_list, configs=FLOOR_CONFIGS):
             tiles = ctx * KV_DIM * 2 // 4096
             if wg > tiles:
                 continue
-            us = sw.us_per_call(lambda f, n: sw.enqueue_floor([ctx], f, n, wg, waves, inflight), reps=2)
+            us = sw.us_per_call(lambda f, n: sw.enqueue_floor([ctx], f, n, wg, waves, inflight), reps=2, steps=n_slices(ctx))
             if best is None or us < best[0]:
                 best = (us, wg, waves, inflight)
         us, wg, waves, inflight = best
@@ -422,7 +431,7 @@ def dispatch_rows(sw, ctx_list):
     rows = []
     for ctx in ctx_list:
         def timed(**over):
-            return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over))
+            return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over), steps=n_slices(ctx))
         timed()  # the first graph timed on a context's slices runs up to a microsecond per call slow: discard one
         auto = timed()
         alts = {}
@@ -444,7 +453,7 @@ def dispatch_rows(sw, ctx_list):
 def per_ctx_rows(sw, ctx_list, replays):
     rows = []
     for ctx in ctx_list:
-        us = sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n), reps=3, replays=replays)
+        us = sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n), reps=3, replays=replays, steps=n_slices(ctx))
         gbs = algorithmic_bytes(ctx, sw.n_q) / (us * 1e-6) / 1e9
         p = sw.plan(ctx)
         rows.append({"ctx": ctx, "us_per_layer": round(us, 3), "GBps": round(gbs, 1), "frac_peak": round(gbs / HBM_PEAK_GBS, 4),
@@ -627,7 +636,8 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%s layer shape (%d Q / 8 KV heads, head_dim 128), batch 1, one decode-"
                                "attention layer call per context in %s per step, bf16 KV cache, %s layout, "
-                               "HIP-graph replays over %d rotating KV slices per context"
+                               "HIP-graph replays over %d rotating KV slices per context (per-context figures: over at "
+                               "least 512 MiB of slices from 1024 positions up, so no length replays out of the 256 MB Infinity Cache)"
                                % ("Qwen3-4B" if n_q == 32 else "Qwen3-32B-heads" if n_q == 64 else "custom", n_q,
                                   ctx_list, layout_name, SLICES),
                    "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout},

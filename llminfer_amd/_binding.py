@@ -151,6 +151,13 @@ def lib():
             raise RuntimeError(
                 "libllmi_hip.so is not built (%s missing); run `python -m llminfer_amd.build`. "
                 "There is no fallback implementation." % LIB_PATH)
+        # PyTorch ships a HIP runtime of its own. When both are in a process, torch's has to be loaded first:
+        # the library then binds to that one, and the device pointers torch hands out are its own. (Loaded the
+        # other way round the process holds two runtimes, and launches fail with "no ROCm-capable device".)
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         for name, (restype, argtypes) in SYMBOLS.items():
             fn = getattr(L, name)
