@@ -19,9 +19,10 @@
 //   * a workgroup serves ALL query heads of its KV head, so K and V are read
 //     from HBM exactly once (the reference re-reads them once per query head,
 //     mha_kernel.cu:67,104);
-//   * K/V tiles stream through per-wave LDS rings filled by LDS-DMA loads; the
-//     query rows (and the append variant's operands) take the same road, issued
-//     ahead of the tiles, so that every wait is a hand-placed vmcnt;
+//   * K/V tiles stream through per-wave LDS rings filled by LDS-DMA loads, every
+//     load instruction a run of whole 256-byte rows (1 KiB of contiguous memory
+//     in the head-major layout); the query rows (and the append variant's operands)
+//     take the same road, issued ahead of the tiles, so that every wait is a hand-placed vmcnt;
 //   * q.K^T runs on the matrix cores: one v_mfma_f32_16x16x32_bf16 chain per
 //     tile of 16 positions, K rows as the A operand (lane = row, no transpose
 //     needed because the contraction over head_dim is order-free), the query
@@ -39,7 +40,10 @@
 //   QK  A  lane L: row r = L%16, dims (j*4 + L/16)*8 .. +8 for step j = 0..3
 //   QK  B  lane L: head h = L%16 (zero for h >= group), same dims
 //   QK  C  lane L: head h = L%16, rows r = 4*(L/16) + i in register i = 0..3
-//   V load lane L: rows r = 4*(L/16) + i (load i), columns (L%16)*8 .. +8
+//   loads  lane L: K and V load i fetch rows 4i + L/16 whole (256 contiguous bytes over the row's 16 lanes;
+//                  K with its 16-byte chunks swizzled by row & 7); the operands are read back from
+//                  LDS in the layouts above and below
+//   V oper lane L: rows r = 4*(L/16) + i (register i), columns (L%16)*8 .. +8
 //   PV  A  lane L: head h = L%16, rows 4*(L/16) + i      (= QK C, as bf16)
 //   PV  B  lane L: rows 4*(L/16) + i, column 8*(L%16) + j for product j = 0..7
 //   PV  C  lane L: heads 4*(L/16) + i, column 8*(L%16) + j (accumulator o[j][i])
@@ -360,9 +364,18 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     const char* vb = reinterpret_cast<const char*>(a.v + (int64_t)kvh * a.head_stride + (int64_t)begin * a.row_stride);
     const uint32_t rs = (uint32_t)a.row_stride * 2u;           // bytes per position step
     const uint32_t last_off = (uint32_t)(nrows - 1) * rs;      // rows past the range clamp to its last row
-    const uint32_t k_row = (uint32_t)n16 * rs;
-    const uint32_t k_col = (uint32_t)kg * 16u;
-    const uint32_t v_row = (uint32_t)(4 * kg) * rs;
+    // K load i of a tile fetches rows 4i .. 4i+3 whole (DPP row kg takes row 4i + kg, 256 contiguous
+    // bytes across its 16 lanes): every request is a full cache line in either layout, and in the
+    // head-major layout one instruction covers 1 KiB of contiguous memory. Lane p of the row fetches
+    // 16-byte chunk p ^ (row & 7): the swizzle that lets the MFMA operand read below (lane = row,
+    // 16 rows 256 bytes apart) spread over the LDS banks instead of hitting one.
+    const uint32_t k_row = (uint32_t)kg * rs;
+    const uint32_t k_col0 = (uint32_t)(n16 ^ kg) * 16u;        // rows 4i + kg with i even: (row & 7) = kg
+    const uint32_t k_col1 = (uint32_t)(n16 ^ (4 + kg)) * 16u;  // i odd: (row & 7) = 4 + kg
+    // Operand read: row n16 sits in load n16 / 4, at row slot n16 % 4; chunk c is at lane slot c ^ (n16 & 7).
+    const uint32_t k_rd = (uint32_t)((n16 >> 2) * 1024 + (n16 & 3) * 256);
+    const uint32_t k_rd0 = k_rd + (uint32_t)((kg ^ (n16 & 7)) * 16);        // chunks j*4 + kg, j even (+ 128 bytes for j = 2)
+    const uint32_t k_rd1 = k_rd + (uint32_t)(((4 + kg) ^ (n16 & 7)) * 16);  // j odd (+ 128 bytes for j = 3)
     const uint32_t v_col = (uint32_t)n16 * 16u;
 
     float m_run = -INFINITY;  // running max, exp2 domain, per (head = n16)
@@ -384,9 +397,10 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
 
     // Each wave streams its tiles through a private ring of NSTAGE LDS slots
     // (8 KiB each: 4 KiB of K rows, 4 KiB of V rows) filled by LDS-DMA loads,
-    // so the bytes in flight cost no VGPRs. A lane later reads back exactly the
-    // 16 bytes it asked for (offset 16*lane inside each 1 KiB load), so the LDS
-    // reads are linear and conflict-free. Out-of-range rows of a ragged last
+    // so the bytes in flight cost no VGPRs. A load lands at offset 16*lane of its
+    // 1 KiB block, i.e. as four whole rows; the operand reads pick their 16 bytes
+    // out of those rows (K through a row-dependent swizzle, V directly), both free
+    // of bank conflicts. Out-of-range rows of a ragged last
     // tile read the last valid row and are masked out of the softmax.
     constexpr int kStageBytes = 8192;
     constexpr int kRingBytes = NW * NSTAGE * kStageBytes;
@@ -423,22 +437,29 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         const uint32_t base = (uint32_t)t * (kTile * rs);
         const uint32_t slot = my_ring_lds + (uint32_t)stage * kStageBytes;
-        const uint32_t ko = min(base + k_row, last_off) + k_col;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(kb, ko + j * 64, slot + j * 1024);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t vo = min(base + v_row + (uint32_t)i * rs, last_off) + v_col;
+            const uint32_t ko = min(base + k_row + (uint32_t)(4 * i) * rs, last_off) + ((i & 1) ? k_col1 : k_col0);
+            dma16(kb, ko, slot + i * 1024);
+        }
+        // V the same way: load i fetches rows 4i .. 4i+3 whole. The operand wants rows 4*kg + i in lane
+        // (kg, n16): row r sits in load r / 4 at row slot r % 4, read back below without bank conflicts
+        // (the 16 lanes of a DPP row read 256 consecutive bytes).
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t vo = min(base + k_row + (uint32_t)(4 * i) * rs, last_off) + v_col;
             dma16(vb, vo, slot + 4096 + i * 1024);
         }
     };
 
     auto read_tile = [&](int stage, TileRegs& r) {
-        const u32x4* sp = reinterpret_cast<const u32x4*>(my_ring + stage * kStageBytes) + lane;
+        const char* kp = my_ring + stage * kStageBytes;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) r.k[j] = sp[j * 64];
+        for (int j = 0; j < 4; ++j)
+            r.k[j] = *reinterpret_cast<const u32x4*>(kp + ((j & 1) ? k_rd1 : k_rd0) + (j >> 1) * 128);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r.v[i] = sp[(4 + i) * 64];
+        for (int i = 0; i < 4; ++i)
+            r.v[i] = *reinterpret_cast<const u32x4*>(kp + 4096 + kg * 1024 + i * 256 + n16 * 16);
     };
 
     auto compute_tile = [&](int t, const TileRegs& r) {
