@@ -24,9 +24,9 @@ thread_local std::string g_last_error;
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
 // memory round trips for its combine, while one workgroup streams a whole KV
-// head of 10 tiles in about 5.2 us: measured at 32 query / 8 KV heads under graph
-// replay, single pass 5.2 vs split 5.9 us at 160 positions, 6.3 vs 6.0 us at 176.)
-constexpr int kSinglePassMaxLen = 160;
+// head of 13 tiles in about 4.9 us: measured at 32 query / 8 KV heads under graph
+// replay, single pass 4.87 vs split 4.95 us at 208 positions, 4.99 vs 4.96 us at 224.)
+constexpr int kSinglePassMaxLen = 208;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).
@@ -109,9 +109,9 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
 
     const int single_waves_max = (max_waves < wave_cap ? max_waves : wave_cap);  // 8 where the kernel variant allows
     // Groups of 8 query heads run 8 waves per workgroup, which carry a single pass a little further
-    // (64 query / 8 KV heads: single pass 4.96 / 5.36 us against 5.47 / 5.61 us split at 176 / 208
-    // positions, 6.30 against 5.71 at 256).
-    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 208 : kSinglePassMaxLen;
+    // (64 query / 8 KV heads: single pass 5.16 / 5.73 us against 5.71 / 5.70 us split at 208 / 288
+    // positions, 5.97 against 5.82 at 320).
+    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 288 : kSinglePassMaxLen;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
@@ -150,7 +150,10 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             // (64 query / 8 KV heads, 16 against 32 splits: 6.13 : 6.94 us at 512 positions, 6.65 : 7.12
             // at 1024, 7.22 : 7.70 at 1500; 32 splits ahead from 2048).
             const int full = target * (waves == 8 ? 4 : 1);
-            want = tiles >= full ? target : tiles >= half ? half : quarter;
+            // (... and half again until a split has a tile and a half: 8 against 16 splits 5.55 : 5.76 us at
+            // 256 positions, 5.70 : 5.84 at 288, level at 352)
+            const int half_from = waves == 8 ? half + half / 2 : half;
+            want = tiles >= full ? target : tiles >= half_from ? half : quarter;
             if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;
             const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
