@@ -146,10 +146,10 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             if (half < 2) half = 2;
             int quarter = half / 2;
             if (quarter < 2) quarter = 2;
-            // With 8 waves per workgroup a split wants four tiles before one workgroup per CU pays
-            // (64 query / 8 KV heads, 16 against 32 splits: 6.13 : 6.94 us at 512 positions, 6.65 : 7.12
-            // at 1024, 7.22 : 7.70 at 1500; 32 splits ahead from 2048).
-            const int full = target * (waves == 8 ? 4 : 1);
+            // With 8 waves per workgroup (one LDS stage per wave) a split wants two tiles per wave before
+            // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.44 : 6.31 us at 512
+            // positions, 6.60 : 7.21 at 2048, level at 8192, 27.6 : 25.0 at 32768).
+            const int full = target * (waves == 8 ? 16 : 1);
             // (... and half again until a split has a tile and a half: 8 against 16 splits 5.55 : 5.76 us at
             // 256 positions, 5.70 : 5.84 at 288, level at 352)
             const int half_from = waves == 8 ? half + half / 2 : half;
