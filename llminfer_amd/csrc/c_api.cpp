@@ -109,9 +109,9 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
 
     const int single_waves_max = (max_waves < wave_cap ? max_waves : wave_cap);  // 8 where the kernel variant allows
     // Groups of 8 query heads run 8 waves per workgroup, which carry a single pass a little further
-    // (64 query / 8 KV heads: single pass 5.16 / 5.73 us against 5.71 / 5.70 us split at 208 / 288
-    // positions, 5.97 against 5.82 at 320).
-    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 288 : kSinglePassMaxLen;
+    // (64 query / 8 KV heads: single pass 5.14 us against 5.64 us split at 208 positions; at 256, where
+    // 16 splits have a tile each, 5.51 against 5.34).
+    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 240 : kSinglePassMaxLen;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
@@ -150,10 +150,7 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.44 : 6.31 us at 512
             // positions, 6.60 : 7.21 at 2048, level at 8192, 27.6 : 25.0 at 32768).
             const int full = target * (waves == 8 ? 16 : 1);
-            // (... and half again until a split has a tile and a half: 8 against 16 splits 5.55 : 5.76 us at
-            // 256 positions, 5.70 : 5.84 at 288, level at 352)
-            const int half_from = waves == 8 ? half + half / 2 : half;
-            want = tiles >= full ? target : tiles >= half_from ? half : quarter;
+            want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;
             const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
