@@ -355,9 +355,15 @@ class Sweep:
 
     def enqueue_floor(self, ctxs, first_step, steps, workgroups, waves, inflight):
         probe = self.B.lib().llmi_hip_probe_stream_read
+        probe_rows = self.B.lib().llmi_hip_probe_stream_read_rows
         for s in range(first_step, first_step + steps):
             for ctx in ctxs:
                 off = self.regions[(ctx, s % n_slices(ctx))] * 2
+                if self.layout == 0:  # position-major: the same bytes as 256-byte pieces of 2 KiB rows, a grid row per KV head
+                    self.B.check(probe_rows(self.k.data_ptr() + off, self.v.data_ptr() + off, ctx, N_KV, max(1, workgroups // N_KV),
+                                            waves, inflight, self.sink.data_ptr(), self.stream.cuda_stream),
+                                 "llmi_hip_probe_stream_read_rows")
+                    continue
                 self.B.check(probe(self.k.data_ptr() + off, self.v.data_ptr() + off, ctx * KV_DIM * 2, workgroups, waves,
                                    inflight, self.sink.data_ptr(), self.stream.cuda_stream), "llmi_hip_probe_stream_read")
 
@@ -667,6 +673,8 @@ def main():
             # the reference's own cache layout (what a maintainer gets who changes nothing but the registry arm)
             sw_pm = Sweep(ctx_list, n_q, 0)
             result["position_major"] = per_ctx_rows(sw_pm, ctx_list, 40)
+            for row, f in zip(result["position_major"], stream_floor(sw_pm, ctx_list)):  # the same pieces, read and thrown away
+                row["stream_floor_us"] = f["us"]
             del sw_pm
             torch.cuda.empty_cache()
             # the dispatch against forced plans at lengths either side of the threshold, powers of two and not

@@ -24,6 +24,13 @@ extern "C" {
 int llmi_hip_probe_stream_read(const void* a, const void* b, size_t bytes_each, int32_t workgroups, int32_t waves,
                                int32_t tiles_in_flight, void* sink, void* stream);
 
+/* The same stream in the position-major cache layout: `a` and `b` hold `rows` rows of `heads` x 256 bytes (a KV head's
+ * part of a row is 256 bytes at offset 256 * head); the grid is (heads, workgroups_per_head), workgroup (h, g) reads head
+ * h's pieces of a contiguous run of 16-row tiles, four rows per load instruction. rows a multiple of 16,
+ * workgroups_per_head <= rows / 16; waves and tiles_in_flight as above. */
+int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, int32_t heads, int32_t workgroups_per_head,
+                                    int32_t waves, int32_t tiles_in_flight, void* sink, void* stream);
+
 /* dst[i] = src[i] for `bytes` bytes (a multiple of 16) with one plain kernel: reads `bytes`, writes `bytes`.
  * The known traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by. */
 int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream);

@@ -81,6 +81,9 @@ class QkNormRopeArgs(ctypes.Structure):
     ]
 
 
+PROBE_PLAIN, PROBE_SC0, PROBE_SC1, PROBE_SC0_SC1, PROBE_NT = range(5)  # llmi_hip_probes.h: cache policy of the hand-over probe
+
+
 class ProbeHandoverResult(ctypes.Structure):
     _fields_ = [(n, ctypes.c_uint32) for n in ("seen", "polls", "ns", "xcc_reader", "xcc_writer")]
 
@@ -125,6 +128,7 @@ SYMBOLS = {
     "llmi_hip_poll_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint64)]),
     # include/llmi_hip_probes.h
     "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
+    "llmi_hip_probe_stream_read_rows": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),

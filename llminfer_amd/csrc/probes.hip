@@ -47,6 +47,42 @@ __global__ __launch_bounds__(NW * 64) void stream_read_kernel(const char* __rest
     if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[0] = acc[0];
 }
 
+// The same stream in the position-major cache layout: the arrays are rows of `row_bytes` bytes, a KV head's part of a row
+// is 256 bytes at offset 256 * head. Workgroup (head, g) reads its head's pieces of a contiguous run of 16-row tiles;
+// a load instruction takes four rows (one per 16 lanes), like the decode kernel's.
+template <int NW, int INFLIGHT>
+__global__ __launch_bounds__(NW * 64) void stream_read_rows_kernel(const char* __restrict__ a, const char* __restrict__ b,
+                                                                   uint32_t tiles, uint32_t row_bytes, uint32_t* sink) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t head = blockIdx.x, g = blockIdx.y, G = gridDim.y;
+    const uint32_t run = tiles / G, longer = tiles % G;
+    const uint32_t first = g * run + (g < longer ? g : longer);
+    const uint32_t count = run + (g < longer ? 1u : 0u);
+    const size_t lane_off = (size_t)(first * 16u + (lane >> 4)) * row_bytes + head * 256u + (lane & 15u) * 16u;
+    const char* pa = a + lane_off;
+    const char* pb = b + lane_off;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (uint32_t t0 = wave; t0 < count; t0 += NW * INFLIGHT) {
+        u32x4 r[INFLIGHT][8];
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+            uint32_t t = t0 + u * NW;
+            if (t >= count) t = t0;  // (a repeat near the end of the run: served by the cache, never out of range)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const size_t off = (size_t)(t * 16u + 4u * j) * row_bytes;
+                r[u][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pa + off));
+                r[u][4 + j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pb + off));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc ^= r[u][j];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[0] = acc[0];
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n16) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
@@ -133,6 +169,17 @@ bool launch_stream(int inflight, dim3 grid, hipStream_t s, const char* a, const 
     }
 }
 
+template <int NW>
+bool launch_stream_rows(int inflight, dim3 grid, hipStream_t s, const char* a, const char* b, uint32_t tiles, uint32_t row_bytes,
+                        uint32_t* sink) {
+    switch (inflight) {
+        case 1: hipLaunchKernelGGL((stream_read_rows_kernel<NW, 1>), grid, dim3(NW * 64), 0, s, a, b, tiles, row_bytes, sink); return true;
+        case 2: hipLaunchKernelGGL((stream_read_rows_kernel<NW, 2>), grid, dim3(NW * 64), 0, s, a, b, tiles, row_bytes, sink); return true;
+        case 4: hipLaunchKernelGGL((stream_read_rows_kernel<NW, 4>), grid, dim3(NW * 64), 0, s, a, b, tiles, row_bytes, sink); return true;
+        default: return false;
+    }
+}
+
 }  // namespace
 }  // namespace llmi
 
@@ -157,6 +204,31 @@ int llmi_hip_probe_stream_read(const void* a, const void* b, size_t bytes_each, 
         case 2: ok = launch_stream<2>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
         case 4: ok = launch_stream<4>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
         case 8: ok = launch_stream<8>(tiles_in_flight, dim3(workgroups), s, pa, pb, tiles, ps); break;
+        default: ok = false;
+    }
+    if (!ok) return LLMI_ERR_INVALID_ARG;
+    return check_launch();
+}
+
+int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, int32_t heads, int32_t workgroups_per_head,
+                                    int32_t waves, int32_t tiles_in_flight, void* sink, void* stream) {
+    if (!a || !b || !sink) return LLMI_ERR_NULL_POINTER;
+    if (rows < 16 || rows % 16 != 0 || heads < 1 || heads > 256) return LLMI_ERR_INVALID_ARG;
+    if (workgroups_per_head < 1 || workgroups_per_head > 65535 || workgroups_per_head > rows / 16) return LLMI_ERR_INVALID_ARG;
+    if (((uintptr_t)a | (uintptr_t)b) & 15u) return LLMI_ERR_ALIGNMENT;
+    const uint32_t tiles = (uint32_t)(rows / 16);
+    const uint32_t row_bytes = (uint32_t)heads * 256u;
+    const char* pa = static_cast<const char*>(a);
+    const char* pb = static_cast<const char*>(b);
+    uint32_t* ps = static_cast<uint32_t*>(sink);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)heads, (unsigned)workgroups_per_head);
+    bool ok = false;
+    switch (waves) {
+        case 1: ok = launch_stream_rows<1>(tiles_in_flight, grid, s, pa, pb, tiles, row_bytes, ps); break;
+        case 2: ok = launch_stream_rows<2>(tiles_in_flight, grid, s, pa, pb, tiles, row_bytes, ps); break;
+        case 4: ok = launch_stream_rows<4>(tiles_in_flight, grid, s, pa, pb, tiles, row_bytes, ps); break;
+        case 8: ok = launch_stream_rows<8>(tiles_in_flight, grid, s, pa, pb, tiles, row_bytes, ps); break;
         default: ok = false;
     }
     if (!ok) return LLMI_ERR_INVALID_ARG;

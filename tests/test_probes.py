@@ -1,0 +1,105 @@
+"""The measurement kernels of the library (include/llmi_hip_probes.h): argument checks without a GPU, and
+on a GPU that every launch shape bench.py uses runs, that the copy kernel copies and that the hand-over
+probe reports what its policies are known to do."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from llminfer_amd import _binding as B
+
+P = 0x1000  # any aligned non-null address: the checks below return before anything is launched
+
+
+def test_stream_read_rejects_bad_arguments():
+    f = B.lib().llmi_hip_probe_stream_read
+    assert f(None, P, 4096, 1, 4, 1, P, None) == B.STATUS["NULL_POINTER"]
+    assert f(P, P, 4096, 1, 4, 1, None, None) == B.STATUS["NULL_POINTER"]
+    assert f(P, P, 0, 1, 4, 1, P, None) == B.STATUS["INVALID_ARG"]
+    assert f(P, P, 4097, 1, 4, 1, P, None) == B.STATUS["INVALID_ARG"]
+    assert f(P, P, 4096, 0, 4, 1, P, None) == B.STATUS["INVALID_ARG"]
+    assert f(P + 8, P, 4096, 1, 4, 1, P, None) == B.STATUS["ALIGNMENT"]
+
+
+def test_stream_read_rows_rejects_bad_arguments():
+    f = B.lib().llmi_hip_probe_stream_read_rows
+    assert f(None, P, 64, 8, 1, 4, 1, P, None) == B.STATUS["NULL_POINTER"]
+    assert f(P, P, 0, 8, 1, 4, 1, P, None) == B.STATUS["INVALID_ARG"]
+    assert f(P, P, 65, 8, 1, 4, 1, P, None) == B.STATUS["INVALID_ARG"]      # rows: whole 16-row tiles
+    assert f(P, P, 64, 0, 1, 4, 1, P, None) == B.STATUS["INVALID_ARG"]
+    assert f(P, P, 64, 8, 5, 4, 1, P, None) == B.STATUS["INVALID_ARG"]      # more workgroups per head than tiles
+    assert f(P, P + 4, 64, 8, 1, 4, 1, P, None) == B.STATUS["ALIGNMENT"]
+
+
+def test_copy_and_handover_reject_bad_arguments():
+    lib = B.lib()
+    assert lib.llmi_hip_probe_copy(None, P, 16, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_copy(P, P, 24, None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_copy(P, P + 4, 16, None) == B.STATUS["ALIGNMENT"]
+    assert lib.llmi_hip_probe_handover(0, 2, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
+    res = B.ProbeHandoverResult()
+    assert lib.llmi_hip_probe_handover(5, 2, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 16, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 8, 0, P + 16, ctypes.byref(res), None) == B.STATUS["ALIGNMENT"]
+
+
+@pytest.fixture(scope="module")
+def dev():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.mark.gpu
+def test_stream_probes_run_every_launch_shape(dev):
+    """Both stream kernels over ragged tile counts (runs that differ by a tile, fewer tiles than wavefronts x tiles
+    in flight): the launches succeed, the sink stays untouched, and the buffers end where the reads end."""
+    import torch
+    lib = B.lib()
+    rows, heads = 16 * 37, 8                       # 37 tiles: no workgroup count below divides it
+    nbytes = rows * heads * 256
+    k = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev)
+    v = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for waves in (1, 2, 4, 8):
+        for inflight in (1, 2, 4):
+            for wg in (1, 3, 8, 37):
+                assert lib.llmi_hip_probe_stream_read_rows(k.data_ptr(), v.data_ptr(), rows, heads, wg, waves, inflight,
+                                                           sink.data_ptr(), stream) == 0
+            for wg in (1, 5, 64, nbytes // 4096):
+                assert lib.llmi_hip_probe_stream_read(k.data_ptr(), v.data_ptr(), nbytes, wg, waves, inflight, sink.data_ptr(),
+                                                      stream) == 0
+    assert lib.llmi_hip_probe_stream_read(k.data_ptr(), v.data_ptr(), nbytes, 4, 3, 1, sink.data_ptr(), stream) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_stream_read_rows(k.data_ptr(), v.data_ptr(), rows, heads, 4, 4, 3, sink.data_ptr(), stream) == B.STATUS["INVALID_ARG"]
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0
+
+
+@pytest.mark.gpu
+def test_copy_probe_copies(dev):
+    import torch
+    src = torch.randint(-2**31, 2**31 - 1, (1 << 20,), dtype=torch.int32, device=dev)
+    dst = torch.zeros_like(src)
+    assert B.lib().llmi_hip_probe_copy(src.data_ptr(), dst.data_ptr(), src.numel() * 4, torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reader", [8, 9])
+def test_handover_probe_device_scope_sees_the_store(dev, reader):
+    """A device-scope (sc1) load sees a device-scope store from another workgroup, on the writer's XCD and on the
+    next one, within the bounded poll budget; the result names the XCDs both sides ran on."""
+    import torch
+    line = torch.zeros(4096 // 4 + 64, dtype=torch.int32, device=dev)
+    base = (line.data_ptr() + 255) & ~255
+    res = torch.zeros(8, dtype=torch.int32, device=dev)
+    rc = B.lib().llmi_hip_probe_handover(B.PROBE_SC1, B.PROBE_SC1, reader, 1, base, res.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    seen, polls, ns, xr, xw = (int(x) for x in res[:5].cpu())
+    assert seen == 1 and 1 <= polls < 4000 and ns > 0
+    assert 0 <= xr < 8 and 0 <= xw < 8
