@@ -25,7 +25,8 @@ thread_local std::string g_last_error;
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
 // memory round trips for its combine, while one workgroup streams a whole KV
 // head of 13 tiles in about 4.9 us: measured at 32 query / 8 KV heads under graph
-// replay, single pass 4.87 vs split 4.95 us at 208 positions, 4.99 vs 4.96 us at 224.)
+// replay, single pass 4.90 vs split 5.03 us at 208 positions, 5.01 vs 5.05 us at 224,
+// 5.28 vs 4.79 us at 256.)
 constexpr int kSinglePassMaxLen = 208;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
@@ -134,10 +135,10 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
         if (want == 0) {
             // Auto: one workgroup per CU (kTargetGroups / kv heads splits) as soon as every split gets
             // a tile of its own; half as many below that, a quarter when even those would be left
-            // without a tile. Measured with 32 query / 8 KV heads: 32 splits against 16 is 5.87 : 5.98 us
-            // at 700 positions, 5.96 : 6.17 at 1024, 6.38 : 6.74 at 1500 and level at 512; 8 splits
-            // against one per tile is 4.88 : 5.05 us at 176 and 4.88 : 5.09 at 208. More, smaller splits
-            // only add partial-result traffic and lengthen the combine (64 splits: +1 us everywhere).
+            // without a tile. Measured with 32 query / 8 KV heads: 32 splits against 16 is 5.23 : 5.28 us
+            // at 700 positions, 5.77 : 5.84 at 1500, 6.70 : 6.76 at 3000, 7.25 : 7.41 at 4096 and within
+            // 1.5 % the other way at 512, 1024 and 2048. More, smaller splits only add partial-result
+            // traffic and lengthen the combine (64 splits: +1 us everywhere).
             // And no more splits than the caller's workspace can hold.
             int target = kTargetGroups / n_kv;
             if (target < 2) target = 2;
@@ -147,8 +148,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             int quarter = half / 2;
             if (quarter < 2) quarter = 2;
             // With 8 waves per workgroup (one LDS stage per wave) a split wants two tiles per wave before
-            // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.44 : 6.31 us at 512
-            // positions, 6.60 : 7.21 at 2048, level at 8192, 27.6 : 25.0 at 32768).
+            // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.55 : 6.42 us at 512
+            // positions, 6.75 : 7.31 at 2048, 8.08 : 8.63 at 4096, level at 8192, 27.2 : 24.9 at 32768).
             const int full = target * (waves == 8 ? 16 : 1);
             want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
