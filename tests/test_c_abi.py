@@ -240,3 +240,40 @@ def test_poll_limit_round_trip():
     assert lib.llmi_hip_set_poll_limit(7) == 1 << 22
     assert lib.llmi_hip_set_poll_limit(-5) == 7
     assert lib.llmi_hip_set_poll_limit(1 << 22) == 0
+
+
+def test_plan_invariants_over_random_arguments():
+    """Whatever the shape, length, workspace and overrides: a plan that comes back LLMI_OK covers every position
+    exactly once, leaves no split without a tile, fits the workspace it was given and names a kernel that exists."""
+    hyp = pytest.importorskip("hypothesis")
+    st = hyp.strategies
+
+    @hyp.settings(max_examples=600, deadline=None, derandomize=True)
+    @hyp.given(kv_mul=st.integers(1, 16), n_kv=st.sampled_from([1, 2, 4, 8, 16]), ctx=st.integers(1, 140000),
+               slack=st.integers(0, 64), force_path=st.integers(0, 3), num_splits=st.sampled_from([0, 0, 0, 1, 2, 3, 7, 32, 200, 256]),
+               waves=st.sampled_from([0, 0, 1, 2, 4, 8]), ws_kib=st.sampled_from([0, 1, 64, 4096, 1 << 17]))
+    def check(kv_mul, n_kv, ctx, slack, force_path, num_splits, waves, ws_kib):
+        a = good_args(pos=ctx - 1, max_seq_len=ctx + slack, kv_mul=kv_mul, kv_dim=128 * n_kv, head_num=kv_mul * n_kv,
+                      force_path=force_path, num_splits=num_splits, waves_per_group=waves,
+                      workspace=0x2000 if ws_kib else 0, workspace_bytes=ws_kib << 10)
+        rc, p = plan(a)
+        if rc != 0:
+            assert rc in (B.STATUS["WORKSPACE"], B.STATUS["INVALID_ARG"])
+            return
+        tiles = (ctx + 15) // 16
+        assert 1 <= p.num_splits <= min(256, tiles)
+        assert p.rows_per_split % 16 == 0 and p.rows_per_split == -(-tiles // p.num_splits) * 16
+        assert (p.num_splits == 1) == (p.path == B.PATH_SINGLE_PASS)
+        assert p.workspace_needed <= (ws_kib << 10) and (p.num_splits == 1) == (p.workspace_needed == 0)
+        assert p.group_pad in (1, 2, 4, 8, 16) and kv_mul <= p.group_pad < 2 * kv_mul
+        assert p.waves_per_group in (1, 2, 4, 8) and p.group_pad * p.waves_per_group <= 64
+        if waves:
+            assert p.waves_per_group == waves
+        if num_splits and force_path != B.PATH_SINGLE_PASS:
+            assert p.num_splits == min(num_splits, tiles)
+        if force_path == B.PATH_SINGLE_PASS:
+            assert p.num_splits == 1
+        if force_path in (B.PATH_SPLIT, B.PATH_SPLIT_FUSED) and p.num_splits > 1:
+            assert p.path == force_path
+
+    check()
