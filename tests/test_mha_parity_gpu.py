@@ -282,3 +282,28 @@ def test_qwen3_32b_head_layout_at_128k(oracle, dev):
             assert plan.path == B.PATH_SPLIT_FUSED and plan.num_splits == 32 and plan.waves_per_group == 8
         else:
             assert plan.num_splits == 256
+
+
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        kv_mul = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16]))
+        n_kv = int(rng.choice([1, 2, 3, 4, 8]))
+        ctx = int(rng.choice([rng.integers(1, 64), rng.integers(64, 400), rng.integers(400, 3000)]))
+        path = int(rng.choice([B.PATH_AUTO, B.PATH_SINGLE_PASS, B.PATH_SPLIT, B.PATH_SPLIT_FUSED]))
+        splits = 0 if path in (B.PATH_AUTO, B.PATH_SINGLE_PASS) else int(rng.choice([0, 2, 3, 5, 11, 16, 37, 64, 256]))
+        max_waves = 64 // (1 << (kv_mul - 1).bit_length())
+        waves = int(rng.choice([w for w in (0, 1, 2, 4, 8) if w <= max_waves]))
+        layers = int(rng.integers(1, 4))
+        cases.append((i, kv_mul, n_kv, ctx, int(rng.integers(0, 40)), layers, int(rng.integers(0, layers)),
+                      int(rng.choice([B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])), path, splits, waves))
+    return cases
+
+
+@pytest.mark.parametrize("i,kv_mul,n_kv,ctx,slack,layers,layer_id,layout,path,splits,waves", _random_cases(48, 20240607))
+def test_random_shapes_against_oracle(oracle, dev, i, kv_mul, n_kv, ctx, slack, layers, layer_id, layout, path, splits, waves):
+    """48 seeded draws over group size (incl. non powers of two), KV head count, length, padding behind the last
+    position, layer, layout, path, split count and wave count: combinations no hand-written case names."""
+    case = synth.make_case(1000 + i, n_q=kv_mul * n_kv, n_kv=n_kv, ctx=ctx, max_seq_len=ctx + slack, layers=layers, layer_id=layer_id)
+    _check(oracle, dev, case, kv_layout=layout, force_path=path, num_splits=splits, waves_per_group=waves)
