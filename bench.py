@@ -484,6 +484,28 @@ def run_calibrate_hbm(args):
     return 0
 
 
+def run_placement(args):
+    """Where the workgroups of a 128 / 256 / 512-workgroup launch with a decode workgroup's footprint land."""
+    import collections
+    import torch
+    from llminfer_amd import _binding as B
+    ids = torch.zeros(2 * 512, dtype=torch.int32, device="cuda:0")
+    rows = []
+    for wgs in (128, 256, 512):
+        for exclusive in (0, 1):
+            ids.zero_()
+            B.check(B.lib().llmi_hip_probe_placement(wgs, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream), "placement probe")
+            torch.cuda.synchronize()
+            a = ids[:2 * wgs].cpu().numpy().astype("uint32").reshape(-1, 2)
+            per_cu = collections.Counter((int(x), (int(h) >> 8) & 0xFF) for x, h in a)
+            per_xcd = collections.Counter(int(x) for x in a[:, 0])
+            rows.append({"workgroups": wgs, "lds_kib": 84 if exclusive else 66, "distinct_cus": len(per_cu), "max_per_cu": max(per_cu.values()),
+                         "per_xcd": [per_xcd.get(i, 0) for i in range(8)]})
+    print(json.dumps({"metric": "placement of workgroups with a decode workgroup's footprint (256 threads, 66 or 84 KiB of LDS, 5 us each)",
+                      "n_gpus": 1, "rows": rows}))
+    return 0
+
+
 def run_handover_probe(args):
     """How a 4-byte value stored by one workgroup becomes visible to a polling workgroup on the same XCD and
     on another one, for every pair of store / load cache policies."""
@@ -526,6 +548,7 @@ def main():
                     help="time a kernel that only reads the same K/V bytes, next to the decode kernel, at every --ctx")
     ap.add_argument("--calibrate-hbm", action="store_true", help="run the copy kernel of known traffic (for rocprofv3 --pmc)")
     ap.add_argument("--handover-probe", action="store_true", help="store/load cache-policy visibility probe between two workgroups")
+    ap.add_argument("--placement", action="store_true", help="which XCD and CU the workgroups of a 128/256/512-workgroup launch land on")
     ap.add_argument("--layout", type=int, default=1, help="1 = head-major (default), 0 = position-major")
     ap.add_argument("--heads", type=int, default=N_Q, help="query heads (32 = Qwen3-4B, 64 = Qwen3-32B head layout)")
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
@@ -563,6 +586,8 @@ def main():
         return run_calibrate_hbm(args)
     if args.handover_probe:
         return run_handover_probe(args)
+    if args.placement:
+        return run_placement(args)
     if args.gemv:
         return run_gemv(args)
     if args.stack:

@@ -35,6 +35,12 @@ int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, 
  * The known traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by. */
 int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream);
 
+/* Where the workgroups of a launch land. `workgroups` (1..4096) workgroups of 256 threads with the LDS footprint of a
+ * decode workgroup (66 KiB; `exclusive` != 0: 84 KiB, more than half a CU's LDS, so that no two share a CU) each write
+ * ids[2*i] = the XCD and ids[2*i+1] = the hardware id register (HW_REG_HW_ID: CU, shader array and shader engine in
+ * bits 8..15) of the CU they run on, and keep that CU for 5 us. `ids`: 2 * workgroups uint32 of device memory. */
+int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* ids, void* stream);
+
 /* Cache policy of one 4-byte load or store of the hand-over probe: the instruction's sc0 / sc1 / nt bits. */
 enum { LLMI_PROBE_PLAIN = 0, LLMI_PROBE_SC0 = 1, LLMI_PROBE_SC1 = 2, LLMI_PROBE_SC0_SC1 = 3, LLMI_PROBE_NT = 4 };
 

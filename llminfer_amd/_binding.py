@@ -131,6 +131,7 @@ SYMBOLS = {
     "llmi_hip_probe_stream_read_rows": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
+    "llmi_hip_probe_placement": (ctypes.c_int, [c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
 }

@@ -133,8 +133,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
         waves = a->waves_per_group ? a->waves_per_group : auto_waves;
         int want = a->num_splits;
         if (want == 0) {
-            // Auto: one workgroup per CU (kTargetGroups / kv heads splits) as soon as every split gets
-            // a tile of its own; half as many below that, a quarter when even those would be left
+            // Auto: one workgroup per CU (kTargetGroups / kv heads splits) once half as many would need more
+            // than a tile per wavefront; half as many below that, a quarter when even those would be left
             // without a tile. Measured with 32 query / 8 KV heads: 32 splits against 16 is 5.23 : 5.28 us
             // at 700 positions, 5.77 : 5.84 at 1500, 6.70 : 6.76 at 3000, 7.25 : 7.41 at 4096 and within
             // 1.5 % the other way at 512, 1024 and 2048. More, smaller splits only add partial-result
@@ -150,7 +150,12 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             // With 8 waves per workgroup (one LDS stage per wave) a split wants two tiles per wave before
             // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.55 : 6.42 us at 512
             // positions, 6.75 : 7.31 at 2048, 8.08 : 8.63 at 4096, level at 8192, 27.2 : 24.9 at 32768).
-            const int full = target * (waves == 8 ? 16 : 1);
+            // With 4 waves the smaller grid keeps the lead while its wavefronts have up to three tiles each: half as
+            // many partials to read back outweighs the shorter runs (32 query / 8 KV heads, 16 against 32 splits:
+            // 4.92 : 5.07 us at 512 positions, 5.26 : 5.35 at 1024, 6.00 : 6.05 at 2048, 6.78 : 6.70 at 3000,
+            // 7.41 : 7.26 at 4096). Some machines run the 256-workgroup grid 0.3-0.4 us slower at every length
+            // and the others as fast as the rest; there the smaller grid leads up to 4096 positions.
+            const int full = waves == 8 ? target * 16 : half * waves * 3 + 1;
             want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;

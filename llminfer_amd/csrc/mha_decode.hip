@@ -1078,7 +1078,7 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
 // A workgroup that has handed its partial results over (every one but the combiners) is idle while the
 // combine runs: it requests its share of the projection's weight rows -- they do not depend on the
 // attention -- and holds them in registers, waits (bounded) for every head's tag of this launch, reads the
-// attention output with device-coherent loads and finishes its rows: dot products, residual add, one
+// attention output (ordinary loads: see below) and finishes its rows: dot products, residual add, one
 // rounding. The weights stream while HBM would otherwise sit idle behind the attention's hand-over.
 // Needs every workgroup of the grid resident at once (the launcher checks the grid against the CU count).
 template <int G, int NW, int NSTAGE>
@@ -1218,7 +1218,7 @@ template <int G, int NW>
 void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stream) {
     // NW * NSTAGE * 8 KiB of ring must fit the LDS budget of one workgroup.
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
-        dim3 grid(n_kv, ka.num_splits);
+    dim3 grid(n_kv, ka.num_splits);
     const bool dyn = ka.pos_dev != nullptr;  // position read at run time: its own instantiation, the static one pays nothing
     if (append) {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);

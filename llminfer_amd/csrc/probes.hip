@@ -147,6 +147,27 @@ __global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe
     }
 }
 
+// Where the workgroups of a launch land: every workgroup (256 threads, LDS bytes of LDS: the footprint of a
+// decode workgroup, or more than half a CU's LDS so that two cannot share a CU) records the XCD and the
+// hardware id register of the CU it runs on, then keeps its CU for hold_ticks of the 100 MHz clock (bounded),
+// so that the whole grid is resident at once like the decode kernel's.
+template <int LDS>
+__global__ __launch_bounds__(256) void placement_kernel(uint32_t* out, uint32_t hold_ticks) {
+    __shared__ char pad[LDS];
+    if (threadIdx.x == 0) {
+        *reinterpret_cast<volatile char*>(pad) = 1;  // (keeps the allocation)
+        uint32_t hw;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+        out[2 * blockIdx.x] = xcc_id();
+        out[2 * blockIdx.x + 1] = hw;
+    }
+    const unsigned long long t0 = wall_clock64();
+    for (int i = 0; i < 100000; ++i) {  // bounded: 100 us at the most with the sleep below
+        if (wall_clock64() - t0 >= hold_ticks) break;
+        __builtin_amdgcn_s_sleep(8);
+    }
+}
+
 typedef void (*HandoverKernel)(uint32_t*, llmi_probe_handover_result*, int, int);
 template <int WM>
 HandoverKernel pick_reader(int rm) {
@@ -241,6 +262,17 @@ int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream) 
     if (((uintptr_t)src | (uintptr_t)dst) & 15u) return LLMI_ERR_ALIGNMENT;
     hipLaunchKernelGGL(copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), bytes / 16);
+    return check_launch();
+}
+
+int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* ids, void* stream) {
+    if (!ids) return LLMI_ERR_NULL_POINTER;
+    if (workgroups < 1 || workgroups > 4096) return LLMI_ERR_INVALID_ARG;
+    if ((uintptr_t)ids & 3u) return LLMI_ERR_ALIGNMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t hold = 500;  // 5 us
+    if (exclusive) hipLaunchKernelGGL((placement_kernel<84 * 1024>), dim3(workgroups), dim3(256), 0, s, ids, hold);
+    else hipLaunchKernelGGL((placement_kernel<66 * 1024>), dim3(workgroups), dim3(256), 0, s, ids, hold);
     return check_launch();
 }
 

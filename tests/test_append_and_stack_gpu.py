@@ -441,7 +441,8 @@ def test_attention_block_stack_matches_the_oracle_chain(oracle, dev, mode):
 
 @pytest.mark.parametrize("n_q,ctx,hidden,want_launches,extra", [
     (32, 4096, 2560, 1, {}),      # Qwen3-4B: 32 splits, 248 worker workgroups, rows dealt 3 / 3 / 2 per wavefront
-    (32, 1500, 2560, 1, {}),
+    (32, 3500, 2560, 1, {}),
+    (32, 1500, 2560, 2, {}),      # 16 splits: 480 worker wavefronts of 3 rows are too few for 2560 rows
     (16, 700, 1024, 1, {}),       # Qwen3-0.6B head layout
     (64, 5000, 640, 2, {}),       # attention output wider than the fused form takes: two launches, same answer
     (32, 100, 2560, 2, {}),       # single pass: nothing idles, two launches

@@ -37,6 +37,10 @@ def test_copy_and_handover_reject_bad_arguments():
     assert lib.llmi_hip_probe_copy(P, P, 24, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_copy(P, P + 4, 16, None) == B.STATUS["ALIGNMENT"]
     assert lib.llmi_hip_probe_handover(0, 2, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_placement(256, 0, None, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_placement(0, 0, P, None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_placement(4097, 0, P, None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_placement(256, 0, P + 2, None) == B.STATUS["ALIGNMENT"]
     res = B.ProbeHandoverResult()
     assert lib.llmi_hip_probe_handover(5, 2, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_handover(0, 2, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
@@ -103,3 +107,20 @@ def test_handover_probe_device_scope_sees_the_store(dev, reader):
     seen, polls, ns, xr, xw = (int(x) for x in res[:5].cpu())
     assert seen == 1 and 1 <= polls < 4000 and ns > 0
     assert 0 <= xr < 8 and 0 <= xw < 8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("exclusive", [0, 1])
+def test_placement_probe_names_a_cu_for_every_workgroup(dev, exclusive):
+    """One workgroup per CU is what the split path's grid counts on: 256 workgroups with a decode workgroup's LDS
+    footprint report their XCD and CU; every XCD takes its share and at least half the grid has a CU of its own
+    (on the boxes measured: all 256)."""
+    import torch
+    ids = torch.zeros(2 * 256, dtype=torch.int32, device=dev)
+    assert B.lib().llmi_hip_probe_placement(256, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    a = ids.cpu().numpy().astype(np.uint32).reshape(-1, 2)
+    assert np.all(a[:, 0] < 16) and np.all(a[:, 1] != 0)
+    cus = {(int(x), (int(h) >> 8) & 0xFF) for x, h in a}
+    assert len(cus) >= 128
+    assert len(set(int(x) for x in a[:, 0])) >= 1
