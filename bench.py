@@ -72,19 +72,23 @@ def make_arena(torch, dev, ctx_list, n_q=N_Q):
 
 
 def kernel_source_blob():
-    """git's blob id of the decode kernel's source (what `git rev-parse HEAD:llminfer_amd/csrc/mha_decode.hip`
-    prints for a committed file), computed from the file itself."""
+    """git's blob ids of the decode kernel's source and of the dispatcher's (what `git rev-parse
+    HEAD:llminfer_amd/csrc/mha_decode.hip` and `...:c_api.cpp` print for committed files), computed from the
+    files themselves and joined by a '+': the kernel and the plan it is launched with decide the traffic."""
     import hashlib
-    data = open(os.path.join(ROOT, "llminfer_amd", "csrc", "mha_decode.hip"), "rb").read()
-    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+    ids = []
+    for name in ("mha_decode.hip", "c_api.cpp"):
+        data = open(os.path.join(ROOT, "llminfer_amd", "csrc", name), "rb").read()
+        ids.append(hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest())
+    return "+".join(ids)
 
 
 def measured_traffic(ctx_list):
     """HBM bytes per launch of the decode kernel over the default sweep, as counted by rocprofv3
     (FETCH_SIZE + WRITE_SIZE, each scaled by a calibration copy): bench.py cannot run the profiler on
     itself, so it reports the figure of the committed counter summary -- only for the workload that
-    summary was taken on, and only while the kernel source is the one it was taken from (the summary
-    names its git blob id); otherwise None."""
+    summary was taken on, and only while the kernel's and the dispatcher's sources are the ones it was taken
+    from (the summary names their git blob ids); otherwise None."""
     if ctx_list != DEFAULT_CTX:
         return None
     path = os.path.join(ROOT, "profiles", "mha_decode_kernel_qwen3-4b_ctx1k-32k_hbm_counters.md")
@@ -322,7 +326,7 @@ def run_stack(args, ctx):
 class Sweep:
     """Decode-attention calls over rotating KV slices, captured into HIP graphs and timed with HIP events."""
 
-    def __init__(self, ctx_list, n_q=N_Q, layout=1):
+    def __init__(self, ctx_list, n_q=N_Q, layout=1, plain_workspace=False):
         import torch
         from llminfer_amd import _binding as B
         from llminfer_amd import ops
@@ -335,9 +339,13 @@ class Sweep:
         self.sink = torch.zeros(64, dtype=torch.int32, device=self.dev)
         self.stream = torch.cuda.Stream()
         self.decode = B.lib().llmi_hip_mha_decode
+        # Set-up, once per workspace allocation, like an engine would do it: which 8 KiB blocks of the workspace lie
+        # near which side of the package (the fused combine keeps its hand-over data in near memory then).
+        self.side = 0 if plain_workspace else ops.workspace_side(self.ws)
 
     def call_args(self, ctx, s, **over):
         off = self.regions[(ctx, s)] * 2
+        over.setdefault("workspace_side", self.side)
         return self.ops.make_mha_args(self.q, self.k.data_ptr() + off, self.v.data_ptr() + off, self.out, self.ws, layer_id=0,
                                       pos=ctx - 1, kv_dim=KV_DIM, kv_mul=self.n_q // N_KV, head_num=self.n_q, head_dim=HEAD_DIM,
                                       max_seq_len=ctx, kv_layout=self.layout, **over)
@@ -521,7 +529,7 @@ def run_handover_probe(args):
                 for ld in range(5):
                     reps = []
                     for _ in range(3):
-                        B.check(B.lib().llmi_hip_probe_handover(st, ld, reader, precache, line.data_ptr(), res_d.data_ptr(),
+                        B.check(B.lib().llmi_hip_probe_handover(st, ld, 0, reader, precache, line.data_ptr(), res_d.data_ptr(),
                                                                torch.cuda.current_stream().cuda_stream), "handover probe")
                         torch.cuda.synchronize()
                         r = res_d.cpu().numpy()
@@ -539,6 +547,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--ctx", type=str, default=",".join(map(str, DEFAULT_CTX)))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--plain-workspace", action="store_true",
+                    help="skip llmi_hip_mha_workspace_side: the fused combine's plain workspace layout, wherever it happens to lie")
     ap.add_argument("--no-extras", action="store_true",
                     help="headline sweep only: skip the stream floor, the position-major layout, BASELINE configs 4 and 5 "
                          "and the dispatch check that the default run appends to its JSON line")
@@ -593,7 +603,7 @@ def main():
     if args.stack:
         return run_stack(args, ctx_list[0])
 
-    sw = Sweep(ctx_list, n_q, args.layout)
+    sw = Sweep(ctx_list, n_q, args.layout, args.plain_workspace)
     layout_name = "head-major" if args.layout == 1 else "position-major"
 
     if args.dispatch_check:
@@ -671,7 +681,8 @@ def main():
                                "least 512 MiB of slices from 1024 positions up, so no length replays out of the 256 MB Infinity Cache)"
                                % ("Qwen3-4B" if n_q == 32 else "Qwen3-32B-heads" if n_q == 64 else "custom", n_q,
                                   ctx_list, layout_name, SLICES),
-                   "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout},
+                   "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout,
+                   "workspace_side": "0x%x" % (sw.side & 0xffffffff)},
         "timed_region_s": round(ms * 1e-3, 6),
         "long_run": {"seconds": round(sum(batch_ms) * 10 * SLICES * 1e-3, 3), "batches": len(batch_ms), "steps_per_batch": 10 * SLICES,
                      "ms_per_step_median": round(median_ms, 6), "value_median": round(step_bytes / (median_ms * 1e-3) / 1e9, 1),

@@ -35,6 +35,14 @@ int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, 
  * The known traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by. */
 int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream);
 
+/* Hand-over latency from every XCD through two blocks of memory. Workgroups i and i + 8 of a grid of 16 (one XCD when
+ * workgroups are dealt to the XCDs in turn) play ping-pong through their own 256-byte line of `a` (2 KiB, 256-byte
+ * aligned, device), then of `b`, twice 16 round trips each, with device-scope stores and polls; every poll loop is
+ * bounded. out[8*i + 0] = the XCD pair i's first workgroup ran on, [1] / [2] = 10 ns ticks spent on a / on b, [3] = 1 if
+ * every number arrived, [5] = the XCD of the pair's second workgroup. `out`: 64 uint32 of device memory. Both blocks and
+ * `out` are overwritten. What llmi_hip_mha_workspace_side decides on. */
+int llmi_hip_probe_block_pingpong(void* a, void* b, uint32_t* out, void* stream);
+
 /* Where the workgroups of a launch land. `workgroups` (1..4096) workgroups of 256 threads with the LDS footprint of a
  * decode workgroup (66 KiB; `exclusive` != 0: 84 KiB, more than half a CU's LDS, so that no two share a CU) each write
  * ids[2*i] = the XCD and ids[2*i+1] = the hardware id register (HW_REG_HW_ID: CU, shader array and shader engine in
@@ -52,13 +60,13 @@ typedef struct llmi_probe_handover_result {
     uint32_t xcc_reader, xcc_writer; /* XCD each side ran on (hardware id register)                        */
 } llmi_probe_handover_result;
 
-/* One writer workgroup (index 0 of 16) stores a value with `store_policy`, one reader workgroup
- * (`reader_workgroup`, 1..15: 8 lands on the writer's XCD, 9 on the next one when workgroups are dealt
- * to the XCDs in turn) polls for it with `load_policy`, a bounded number of times. With `precache` the reader
- * has read the line before the writer writes, so stale copies exist in its L1 and L2. `line` is 4 KiB of
- * device scratch, `result` device memory; both are overwritten. Every loop in the kernel is bounded. */
-int llmi_hip_probe_handover(int32_t store_policy, int32_t load_policy, int32_t reader_workgroup, int32_t precache,
-                            void* line, llmi_probe_handover_result* result, void* stream);
+/* One writer workgroup (`writer_workgroup`, 0..15, of a grid of 16) stores a value with `store_policy`, one reader
+ * workgroup (`reader_workgroup`, 0..15, another one) polls for it with `load_policy`, a bounded number of times. When
+ * workgroups are dealt to the XCDs in turn, workgroups w and w + 8 share an XCD and w + 1 is on the next one. With
+ * `precache` the reader has read the line before the writer writes, so stale copies exist in its L1 and L2. `line` is
+ * 4 KiB of device scratch, `result` device memory; both are overwritten. Every loop in the kernel is bounded. */
+int llmi_hip_probe_handover(int32_t store_policy, int32_t load_policy, int32_t writer_workgroup, int32_t reader_workgroup,
+                            int32_t precache, void* line, llmi_probe_handover_result* result, void* stream);
 
 #ifdef __cplusplus
 }

@@ -31,7 +31,7 @@ class MhaArgs(ctypes.Structure):
         ("layer_id", c_i32), ("pos", c_i32), ("kv_dim", c_i32), ("kv_mul", c_i32),
         ("head_num", c_i32), ("head_dim", c_i32), ("max_seq_len", c_i32), ("kv_layout", c_i32),
         ("force_path", c_i32), ("num_splits", c_i32), ("waves_per_group", c_i32),
-        ("stream", c_void_p), ("pos_device", c_void_p),
+        ("stream", c_void_p), ("pos_device", c_void_p), ("workspace_side", c_i32),
     ]
 
 
@@ -66,7 +66,7 @@ GEMV_OUT_BF16, GEMV_OUT_F32, GEMV_ADD_BF16 = 0, 1, 2
 class MhaPlan(ctypes.Structure):
     _fields_ = [
         ("path", c_i32), ("num_splits", c_i32), ("rows_per_split", c_i32),
-        ("waves_per_group", c_i32), ("group_pad", c_i32), ("workspace_needed", c_size_t),
+        ("waves_per_group", c_i32), ("group_pad", c_i32), ("workspace_side", c_i32), ("workspace_needed", c_size_t),
     ]
 
 
@@ -107,6 +107,7 @@ SYMBOLS = {
     "llmi_hip_mha_decode_append_oproj": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
     "llmi_hip_mha_oproj_launches": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
     "llmi_hip_mha_workspace_bytes": (c_size_t, [c_i32, c_i32, c_i32]),
+    "llmi_hip_mha_workspace_side": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, ctypes.POINTER(c_i32)]),
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),
     "llmi_hip_sincos_table": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_void_p]),
     "llmi_hip_kv_restride": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p]),
@@ -130,8 +131,9 @@ SYMBOLS = {
     "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_stream_read_rows": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
-    "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
+    "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_probe_placement": (ctypes.c_int, [c_i32, c_i32, c_void_p, c_void_p]),
+    "llmi_hip_probe_block_pingpong": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
 }

@@ -150,12 +150,13 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             // With 8 waves per workgroup (one LDS stage per wave) a split wants two tiles per wave before
             // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.55 : 6.42 us at 512
             // positions, 6.75 : 7.31 at 2048, 8.08 : 8.63 at 4096, level at 8192, 27.2 : 24.9 at 32768).
-            // With 4 waves the smaller grid keeps the lead while its wavefronts have up to three tiles each: half as
-            // many partials to read back outweighs the shorter runs (32 query / 8 KV heads, 16 against 32 splits:
-            // 4.92 : 5.07 us at 512 positions, 5.26 : 5.35 at 1024, 6.00 : 6.05 at 2048, 6.78 : 6.70 at 3000,
-            // 7.41 : 7.26 at 4096). Some machines run the 256-workgroup grid 0.3-0.4 us slower at every length
-            // and the others as fast as the rest; there the smaller grid leads up to 4096 positions.
-            const int full = waves == 8 ? target * 16 : half * waves * 3 + 1;
+            // With 4 waves the smaller grid keeps the lead while its wavefronts have up to three tiles each (two in the
+            // position-major layout): half as many partials to read back outweighs the shorter runs. 32 query / 8 KV
+            // heads, workspace laid out by package side, 16 against 32 splits: 5.23 : 5.42 us at 1024 positions,
+            // 5.96 : 6.13 at 2048, 6.70 : 6.79 at 3000, 7.31 : 7.38 at 4096, 8.01 : 7.96 at 5000, 10.16 : 9.65 at 8192;
+            // position-major 6.12 : 6.18 at 2048, 7.16 : 7.05 at 3000, 7.85 : 7.59 at 4096.
+            const int per_wave = a->kv_layout == LLMI_KV_LAYOUT_HEAD_MAJOR ? 3 : 2;
+            const int full = waves == 8 ? target * 16 : half * waves * per_wave + 1;
             want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
             const size_t per_split = fused ? per_split_fused : per_split_plain;
@@ -188,9 +189,23 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
     p->rows_per_split = tiles_per_split * kTile;
     p->waves_per_group = waves;
     p->group_pad = group_pad;
+    p->workspace_side = 0;
     p->workspace_needed = num_splits <= 1 ? 0
                           : path == LLMI_PATH_SPLIT_FUSED ? per_split_fused * (size_t)num_splits + 16
                                                           : per_split_plain * (size_t)num_splits;
+    // The workspace laid out by package side: where every split of a KV head and its combiner run on one XCD (the KV
+    // head is the fastest grid index and the head count a multiple of the eight XCDs), where one wavefront merges
+    // a head (the shared read-back of larger groups keeps the plain layout), and where the workspace has room
+    // for two homes per row, rounded to whole 8 KiB blocks, behind the way to the next 16 KiB boundary. Otherwise the
+    // plain layout, silently: the side only ever changes the time.
+    if (path == LLMI_PATH_SPLIT_FUSED && num_splits > 1 && a->workspace_side != 0 && n_kv % 8 == 0 && a->kv_mul <= waves &&
+        a->head_num <= 128) {
+        const size_t need = side_pad(a->workspace) + fused_workspace(a->head_num, a->head_dim, num_splits, true).bytes();
+        if (a->workspace_bytes >= need) {
+            p->workspace_side = 1;
+            p->workspace_needed = need;
+        }
+    }
     return LLMI_OK;
 }
 
@@ -231,6 +246,33 @@ int llmi_hip_mha_decode_static(const llmi_mha_args* args) {
     if (plan.workspace_needed > bytes) return LLMI_ERR_WORKSPACE;  // (make_plan has checked this already)
     a.workspace = ptr;
     a.workspace_bytes = bytes;
+    // The array's package side, measured once per device: on the first call that is not being captured.
+    {
+        constexpr int kMaxDevices = 64;
+        static std::atomic<int> measured[kMaxDevices];
+        static std::atomic<int32_t> sides_of[kMaxDevices];
+        int dev = 0;
+        if (int rc = record_hip_error(hipGetDevice(&dev), "hipGetDevice")) return rc;
+        int32_t sides = 0;
+        if (dev >= 0 && dev < kMaxDevices) {
+            if (measured[dev].load(std::memory_order_acquire)) {
+                sides = sides_of[dev].load(std::memory_order_relaxed);
+            } else {
+                hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+                hipStream_t s = static_cast<hipStream_t>(a.stream);
+                if (hipStreamIsCapturing(s, &cs) == hipSuccess && cs == hipStreamCaptureStatusNone) {
+                    if (int rc = measure_workspace_side(ptr, bytes, s, &sides)) return rc;
+                    sides_of[dev].store(sides, std::memory_order_relaxed);
+                    measured[dev].store(1, std::memory_order_release);
+                } else {
+                    (void)hipGetLastError();  // (this call only: the plain layout)
+                }
+            }
+        }
+        a.workspace_side = sides;
+        if (a.workspace_side != args->workspace_side)
+            if (int rc = make_plan(&a, &plan)) return rc;  // (same plan, now with the side's layout if it fits)
+    }
     return launch_mha_decode(a, plan);
 }
 
@@ -266,11 +308,7 @@ static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, boo
     int32_t rows_per_wave = 0, max_k = 0;
     oproj_limits(&rows_per_wave, &max_k);
     const int64_t k = (int64_t)m.head_num * m.head_dim;
-    if (plan->path != LLMI_PATH_SPLIT_FUSED || plan->num_splits < 2 || m.pos_device) return LLMI_OK;
-    if (plan->group_pad > 8 || plan->waves_per_group != (plan->group_pad == 8 ? 8 : 4)) return LLMI_OK;
-    if (k % 512 != 0 || k > max_k) return LLMI_OK;
-    const int64_t worker_waves = (int64_t)n_kv * (plan->num_splits - 1) * plan->waves_per_group;
-    if (args->hidden > rows_per_wave * worker_waves) return LLMI_OK;
+    if (m.pos_device || k % 512 != 0 || k > max_k || m.head_num > 128) return LLMI_OK;  // (one wavefront collects the heads' tags, two per lane)
     // every workgroup must be resident at once: the workers wait for the combiners
     static std::atomic<int> cu_count{0};
     int cus = cu_count.load(std::memory_order_relaxed);
@@ -282,10 +320,30 @@ static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, boo
         }
         cu_count.store(cus, std::memory_order_relaxed);
     }
-    if ((int64_t)n_kv * plan->num_splits > cus) return LLMI_OK;
-    if (m.head_num > 128) return LLMI_OK;  // one wavefront collects the heads' tags, two per lane
-    if (m.workspace_bytes < plan->workspace_needed + (size_t)m.head_num * sizeof(uint32_t)) return LLMI_OK;
-    *fused = true;
+    auto fits = [&](const llmi_mha_plan& p) {
+        if (p.path != LLMI_PATH_SPLIT_FUSED || p.num_splits < 2) return false;
+        if (p.group_pad > 8 || p.waves_per_group != (p.group_pad == 8 ? 8 : 4)) return false;
+        const int64_t worker_waves = (int64_t)n_kv * (p.num_splits - 1) * p.waves_per_group;
+        if (args->hidden > rows_per_wave * worker_waves) return false;
+        if ((int64_t)n_kv * p.num_splits > cus) return false;
+        return m.workspace_bytes >= p.workspace_needed + (size_t)m.head_num * sizeof(uint32_t);
+    };
+    if (fits(*plan)) {
+        *fused = true;
+        return LLMI_OK;
+    }
+    // The dispatcher's own split count may leave too few idle wavefronts for the rows (it prefers half a grid up to
+    // four tiles per wavefront): the one-launch form then asks for one workgroup per CU itself.
+    if (m.num_splits == 0 && m.force_path != LLMI_PATH_SINGLE_PASS && plan->num_splits > 1 && cus / n_kv > plan->num_splits) {
+        llmi_mha_args wide = m;
+        wide.num_splits = cus / n_kv > kMaxSplits ? kMaxSplits : cus / n_kv;
+        wide.force_path = LLMI_PATH_SPLIT_FUSED;
+        llmi_mha_plan p2;
+        if (make_plan(&wide, &p2, kMaxWaves, 1) == LLMI_OK && p2.num_splits == wide.num_splits && fits(p2)) {
+            *plan = p2;
+            *fused = true;
+        }
+    }
     return LLMI_OK;
 }
 
@@ -316,8 +374,24 @@ size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t 
     // Per head and split: head_dim partial outputs plus either (max, sum) as two floats
     // (separate combine kernel) or two 8-byte arrival records (fused combine).
     // ... and, behind the records, one 4-byte counter per head for the fused output projection.
-    return (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16 +
-           (size_t)head_num * sizeof(uint32_t);
+    // ... and room for the layout by package side: the way to the first 8 KiB boundary, both arrays rounded up to whole
+    // blocks per side; never less than what llmi_hip_mha_workspace_side needs for its measurement.
+    const size_t plain = (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16;
+    const size_t by_side = fused_workspace(head_num, head_dim, splits, true).bytes() + 2 * kSideBlock;
+    size_t need = (plain > by_side ? plain : by_side) + (size_t)head_num * sizeof(uint32_t);
+    if (need < 6 * kSideBlock) need = 6 * kSideBlock;
+    return need;
+}
+
+int llmi_hip_mha_workspace_side(void* workspace, size_t workspace_bytes, void* stream, int32_t* side) {
+    if (!workspace || !side) return LLMI_ERR_NULL_POINTER;
+    if (!aligned16(workspace)) return LLMI_ERR_ALIGNMENT;
+    if (workspace_bytes < 6 * kSideBlock) return LLMI_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (int rc = record_hip_error(hipStreamIsCapturing(s, &cs), "hipStreamIsCapturing")) return rc;
+    if (cs != hipStreamCaptureStatusNone) return LLMI_ERR_INVALID_ARG;
+    return measure_workspace_side(workspace, workspace_bytes, s, side);
 }
 
 int llmi_hip_qk_norm_rope_append(const llmi_qk_norm_rope_args* a) {

@@ -151,6 +151,7 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
         m.waves_per_group = o.waves_per_group;
         m.stream = stream();
         m.pos_device = follow_device_pos ? pos_dev_.ptr<int32_t>() : nullptr;
+        m.workspace_side = kernel::workspace_side_of(m.workspace, m.workspace_bytes, stream());  // (measured once, before any capture)
         int rc;
         if (mode == kFusedAppend || block) {
             llmi_mha_append_args f{};
@@ -206,6 +207,10 @@ void DecodeStack::capture(int32_t pos, int32_t mode, bool follow_device_pos) {
     if (graph_) {
         HIP_OK(hipGraphDestroy(graph_));
         graph_ = nullptr;
+    }
+    {   // the workspace's sides cannot be measured under capture: do it now if it has not been done
+        tensor::Tensor& ws = buffers_->get_buffer(ModelBufferType::KVSplitOutput);
+        (void)kernel::workspace_side_of(ws.ptr<float>(), ws.byte_size(), stream());
     }
     HIP_OK(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
     try {

@@ -1,5 +1,9 @@
 #include "kernel_interface.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "llmi_hip.h"
 
 namespace kernel {
@@ -64,6 +68,19 @@ static void fail_on(int rc, const char* what) {
         LLMI_FATAL(what << " failed with status " << rc << " (" << llmi_hip_strerror(rc) << ") " << llmi_hip_last_error());
 }
 
+int32_t workspace_side_of(const void* workspace, size_t bytes, void* stream) {
+    static std::mutex mu;
+    static std::map<const void*, std::pair<size_t, int32_t>> known;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = known.find(workspace);
+    if (it != known.end() && it->second.first == bytes) return it->second.second;
+    int32_t sides = 0;
+    if (llmi_hip_mha_workspace_side(const_cast<void*>(workspace), bytes, stream, &sides) != LLMI_OK)
+        return 0;  // under capture, or too small to measure: the plain layout this time, nothing remembered
+    known[workspace] = {bytes, sides};
+    return sides;
+}
+
 void mha_kernel_hip(const tensor::Tensor& query, const tensor::Tensor& key_cache, const tensor::Tensor& value_cache,
                     const tensor::Tensor& kv_split_output, const tensor::Tensor& output, int32_t layer_id,
                     int32_t pos, int32_t kv_dim, int32_t kv_mul, int32_t head_num, int32_t head_dim,
@@ -104,6 +121,7 @@ void mha_kernel_hip(const tensor::Tensor& query, const tensor::Tensor& key_cache
     a.num_splits = o.num_splits;
     a.waves_per_group = o.waves_per_group;
     a.stream = stream;
+    a.workspace_side = workspace_side_of(a.workspace, a.workspace_bytes, stream);
     fail_on(llmi_hip_mha_decode(&a), "llmi_hip_mha_decode");
 }
 

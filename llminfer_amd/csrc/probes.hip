@@ -117,7 +117,7 @@ constexpr uint32_t kProbePolls = 4000u;
 
 // line[0]: the data word; line[64] (another 256-byte line): reader -> writer "I am polling".
 template <int WM, int RM>
-__global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe_handover_result* res, int reader_wg, int precache) {
+__global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe_handover_result* res, int writer_wg, int reader_wg, int precache) {
     if (threadIdx.x != 0) return;
     uint32_t* data = line;
     uint32_t* flag = line + 64;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe
         res->polls = polls;
         res->ns = (uint32_t)((t1 - t0) * 10ull);
         res->xcc_reader = xcc_id();
-    } else if (blockIdx.x == 0) {
+    } else if ((int)blockIdx.x == writer_wg) {
         res->xcc_writer = xcc_id();
         for (int i = 0; i < 200000; ++i)  // bounded: the reader raises the flag at once
             if (load_policy<LLMI_PROBE_SC1>(flag) == 1u) break;
@@ -168,7 +168,48 @@ __global__ __launch_bounds__(256) void placement_kernel(uint32_t* out, uint32_t 
     }
 }
 
-typedef void (*HandoverKernel)(uint32_t*, llmi_probe_handover_result*, int, int);
+// Hand-over latency from every XCD through two blocks of memory. Workgroups i and i + 8 of a grid of 16 (one XCD when
+// workgroups are dealt to the XCDs in turn) play ping-pong through two words of their own 256-byte line in block `a`,
+// then in block `b`, twice each: i stores a number (device scope), i + 8 polls for it and stores it into the second
+// word, i polls for that. kPingPongs round trips per chain; every poll loop is bounded, a pair that loses a number
+// gives up and says so. Workgroup i < 8 reports: its XCD, its partner's, the ticks (10 ns) spent on a and on b, 1 if
+// every number arrived.
+constexpr int kPingPongs = 16, kPingPongChains = 2, kPingPongPolls = 4000;
+__global__ __launch_bounds__(64) void block_pingpong_kernel(uint32_t* a, uint32_t* b, uint32_t* out) {
+    if (threadIdx.x != 0) return;
+    const int pair = blockIdx.x & 7;
+    const bool leader = blockIdx.x < 8;
+    uint32_t* xcc_partner = out + 8 * pair + 5;  // (written by the partner, plainly: read by the host only)
+    if (!leader) *xcc_partner = xcc_id();
+    unsigned long long t[2] = {0, 0};
+    uint32_t ok = 1, seq = 0;
+    for (int c = 0; c < kPingPongChains && ok; ++c)
+        for (int which = 0; which < 2 && ok; ++which) {
+            uint32_t* line = (which ? b : a) + pair * 64;  // this pair's 256 bytes of the block
+            uint32_t* ping = line;
+            uint32_t* pong = line + 16;
+            const unsigned long long t0 = wall_clock64();
+            for (int i = 0; i < kPingPongs && ok; ++i) {
+                ++seq;
+                uint32_t* mine = leader ? ping : pong;
+                const uint32_t* theirs = leader ? pong : ping;
+                if (leader) store_policy<LLMI_PROBE_SC1>(mine, seq);
+                int polls = 0;
+                while (polls < kPingPongPolls && load_policy<LLMI_PROBE_SC1>(theirs) != seq) ++polls;
+                if (polls == kPingPongPolls) ok = 0;
+                if (!leader) store_policy<LLMI_PROBE_SC1>(mine, seq);
+            }
+            t[which] += wall_clock64() - t0;
+        }
+    if (leader) {
+        out[8 * pair + 0] = xcc_id();
+        out[8 * pair + 1] = (uint32_t)t[0];
+        out[8 * pair + 2] = (uint32_t)t[1];
+        out[8 * pair + 3] = ok;
+    }
+}
+
+typedef void (*HandoverKernel)(uint32_t*, llmi_probe_handover_result*, int, int, int);
 template <int WM>
 HandoverKernel pick_reader(int rm) {
     switch (rm) {
@@ -202,6 +243,66 @@ bool launch_stream_rows(int inflight, dim3 grid, hipStream_t s, const char* a, c
 }
 
 }  // namespace
+}  // namespace llmi
+
+namespace llmi {
+
+// Which 8 KiB blocks lie near which side of the package, seen from the workspace itself: the time of hand-overs between
+// two workgroups of one XCD (block_pingpong_kernel, all eight XCDs at once, each pair reporting the XCD it ran on)
+// through a block with address bit 13 clear and through its neighbour with the bit set. The two sides of the package
+// must disagree about which block is nearer, each clearly: anything else is reported as "no statement" (0).
+static int measure_window_side(char* window, hipStream_t stream, int* side) {
+    *side = 0;
+    // The pairs' lines: the first 2 KiB of either block; the results: the second 4 KiB of the first block.
+    uint32_t* out = reinterpret_cast<uint32_t*>(window + 4096);
+    for (int attempt = 0; attempt < 3; ++attempt) {
+        if (int rc = llmi_hip_probe_block_pingpong(window, window + kSideBlock, out, stream)) return rc;
+        uint32_t r[8][8];
+        if (int rc = record_hip_error(hipMemcpyAsync(r, out, sizeof(r), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync")) return rc;
+        if (int rc = record_hip_error(hipStreamSynchronize(stream), "hipStreamSynchronize")) return rc;
+        long long diff[2] = {0, 0};  // per side of the package: ticks through the clear block minus ticks through the set block
+        int n[2] = {0, 0};
+        for (int p = 0; p < 8; ++p) {
+            if (!r[p][3] || r[p][0] != r[p][5]) continue;  // a pair that lost a number, or did not share an XCD
+            const int sd = (int)(r[p][0] >> 2) & 1;
+            diff[sd] += (long long)r[p][1] - (long long)r[p][2];
+            ++n[sd];
+        }
+        if (n[0] < 2 || n[1] < 2) continue;
+        // Per hand-over (two per round trip), in ns (a tick is 10 ns).
+        const long long handovers = 2ll * kPingPongs * kPingPongChains;
+        const long long d0 = diff[0] * 10 / (n[0] * handovers), d4 = diff[1] * 10 / (n[1] * handovers);
+        constexpr long long kThresholdNs = 25;
+        if (d0 <= -kThresholdNs && d4 >= kThresholdNs) *side = 1;       // XCDs 0-3 are nearer to the clear block, 4-7 to the set one
+        else if (d0 >= kThresholdNs && d4 <= -kThresholdNs) *side = 2;
+        if (*side) break;
+    }
+    return LLMI_OK;
+}
+
+// One window per 2 MiB-aligned region the workspace reaches into: the first 16 KiB-aligned 16 KiB of the region that
+// lie inside the workspace.
+int measure_workspace_side(void* workspace, size_t bytes, hipStream_t stream, int32_t* sides) {
+    *sides = 0;
+    const uintptr_t w0 = reinterpret_cast<uintptr_t>(workspace), w1 = w0 + bytes;
+    uint32_t word = 0;
+    bool any = false;
+    for (uintptr_t i = 0; i < 16; ++i) {
+        const uintptr_t region = ((w0 >> 21) + i) << 21;
+        if (region >= w1) break;
+        uintptr_t window = region > w0 ? region : w0;
+        window = (window + 2 * kSideBlock - 1) & ~(uintptr_t)(2 * kSideBlock - 1);
+        if (window + 2 * kSideBlock > w1 || window + 2 * kSideBlock > region + (1u << 21)) continue;
+        int side = 0;
+        if (int rc = measure_window_side(reinterpret_cast<char*>(window), stream, &side)) return rc;
+        word |= (uint32_t)side << (2 * i);
+        any = true;
+    }
+    if (!any) return LLMI_ERR_WORKSPACE;
+    *sides = (int32_t)word;
+    return LLMI_OK;
+}
+
 }  // namespace llmi
 
 using namespace llmi;
@@ -265,6 +366,19 @@ int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream) 
     return check_launch();
 }
 
+int llmi_hip_probe_block_pingpong(void* a, void* b, uint32_t* out, void* stream) {
+    if (!a || !b || !out) return LLMI_ERR_NULL_POINTER;
+    if (((uintptr_t)a | (uintptr_t)b) & 255u) return LLMI_ERR_ALIGNMENT;
+    if ((uintptr_t)out & 3u) return LLMI_ERR_ALIGNMENT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // (numbers start at 1: the lines and the result start from zero)
+    if (int rc = record_hip_error(hipMemsetAsync(a, 0, 2048, s), "hipMemsetAsync")) return rc;
+    if (int rc = record_hip_error(hipMemsetAsync(b, 0, 2048, s), "hipMemsetAsync")) return rc;
+    if (int rc = record_hip_error(hipMemsetAsync(out, 0, 64 * sizeof(uint32_t), s), "hipMemsetAsync")) return rc;
+    hipLaunchKernelGGL(block_pingpong_kernel, dim3(16), dim3(64), 0, s, static_cast<uint32_t*>(a), static_cast<uint32_t*>(b), out);
+    return check_launch();
+}
+
 int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* ids, void* stream) {
     if (!ids) return LLMI_ERR_NULL_POINTER;
     if (workgroups < 1 || workgroups > 4096) return LLMI_ERR_INVALID_ARG;
@@ -276,11 +390,12 @@ int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* id
     return check_launch();
 }
 
-int llmi_hip_probe_handover(int32_t store_pol, int32_t load_pol, int32_t reader_workgroup, int32_t precache, void* line,
+int llmi_hip_probe_handover(int32_t store_pol, int32_t load_pol, int32_t writer_workgroup, int32_t reader_workgroup, int32_t precache, void* line,
                             llmi_probe_handover_result* result, void* stream) {
     if (!line || !result) return LLMI_ERR_NULL_POINTER;
     if (store_pol < 0 || store_pol > LLMI_PROBE_NT || load_pol < 0 || load_pol > LLMI_PROBE_NT) return LLMI_ERR_INVALID_ARG;
-    if (reader_workgroup < 1 || reader_workgroup > 15) return LLMI_ERR_INVALID_ARG;
+    if (writer_workgroup < 0 || writer_workgroup > 15 || reader_workgroup < 0 || reader_workgroup > 15 || writer_workgroup == reader_workgroup)
+        return LLMI_ERR_INVALID_ARG;
     if ((uintptr_t)line & 255u) return LLMI_ERR_ALIGNMENT;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (int rc = record_hip_error(hipMemsetAsync(line, 0, 4096, s), "hipMemsetAsync")) return rc;
@@ -293,7 +408,7 @@ int llmi_hip_probe_handover(int32_t store_pol, int32_t load_pol, int32_t reader_
         case LLMI_PROBE_SC0_SC1: k = pick_reader<LLMI_PROBE_SC0_SC1>(load_pol); break;
         default: k = pick_reader<LLMI_PROBE_NT>(load_pol); break;
     }
-    hipLaunchKernelGGL(k, dim3(16), dim3(64), 0, s, static_cast<uint32_t*>(line), result, (int)reader_workgroup, (int)precache);
+    hipLaunchKernelGGL(k, dim3(16), dim3(64), 0, s, static_cast<uint32_t*>(line), result, (int)writer_workgroup, (int)reader_workgroup, (int)precache);
     return check_launch();
 }
 

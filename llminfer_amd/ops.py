@@ -36,7 +36,7 @@ def workspace_bytes(head_num, head_dim, max_seq_len):
 
 def make_mha_args(query, key_cache, value_cache, output, workspace, *, layer_id, pos, kv_dim, kv_mul,
                   head_num, head_dim, max_seq_len, kv_layout=B.KV_LAYOUT_POS_MAJOR, force_path=B.PATH_AUTO,
-                  num_splits=0, waves_per_group=0, output_f32=None, stream=None, pos_device=None):
+                  num_splits=0, waves_per_group=0, output_f32=None, stream=None, pos_device=None, workspace_side=0):
     """Fills an llmi_mha_args from torch tensors (or raw integer addresses)."""
     def addr(x):
         return x if (x is None or isinstance(x, int)) else x.data_ptr()
@@ -59,7 +59,19 @@ def make_mha_args(query, key_cache, value_cache, output, workspace, *, layer_id,
     a.kv_layout, a.force_path, a.num_splits, a.waves_per_group = kv_layout, force_path, num_splits, waves_per_group
     a.stream = stream
     a.pos_device = addr(pos_device)
+    a.workspace_side = workspace_side
     return a
+
+
+def workspace_side(workspace, stream=None):
+    """Which 8 KiB blocks of `workspace` lie near which side of the package (llmi_hip_mha_workspace_side): 0, 1 or 2,
+    to be passed as workspace_side with this workspace. Overwrites its first 32 KiB and synchronises the stream."""
+    _check_dev("workspace", workspace, (torch.float32,))
+    side = ctypes.c_int32(0)
+    s = stream if stream is not None else torch.cuda.current_stream(workspace.device).cuda_stream
+    B.check(B.lib().llmi_hip_mha_workspace_side(workspace.data_ptr(), workspace.numel() * workspace.element_size(), s,
+                                                ctypes.byref(side)), "llmi_hip_mha_workspace_side")
+    return side.value
 
 
 def mha_plan(args):

@@ -21,7 +21,7 @@ def from_dev_bf16(t):
 
 
 def run_hip(case, dev, *, kv_layout=B.KV_LAYOUT_POS_MAJOR, force_path=B.PATH_AUTO, num_splits=0,
-            waves_per_group=0, workspace_bytes=None, want_plan=False):
+            waves_per_group=0, workspace_bytes=None, want_plan=False, workspace_side=0, workspace_offset=0):
     """Runs llmi_hip_mha_decode on a case from synth.make_case. Returns (bf16 out as f32, f32 tap[, plan])."""
     n_kv = case["kv_dim"] // case["head_dim"]
     k, v = case["k"], case["v"]
@@ -33,11 +33,15 @@ def run_hip(case, dev, *, kv_layout=B.KV_LAYOUT_POS_MAJOR, force_path=B.PATH_AUT
     out32 = torch.full((case["head_num"] * case["head_dim"],), float("nan"), dtype=torch.float32, device=dev)
     if workspace_bytes is None:
         workspace_bytes = ops.workspace_bytes(case["head_num"], case["head_dim"], case["max_seq_len"])
-    ws = torch.full((max(workspace_bytes // 4, 4),), float("nan"), dtype=torch.float32, device=dev)
+    ws = torch.full((max(workspace_bytes // 4, 4) + workspace_offset // 4,), float("nan"), dtype=torch.float32, device=dev)
+    ws = ws[workspace_offset // 4:]
+    if workspace_side == "measure":  # what an engine does once per workspace; the measurement overwrites part of it
+        workspace_side = ops.workspace_side(ws)
+        ws.fill_(float("nan"))
     scal = dict(layer_id=case["layer_id"], pos=case["pos"], kv_dim=case["kv_dim"], kv_mul=case["kv_mul"],
                 head_num=case["head_num"], head_dim=case["head_dim"], max_seq_len=case["max_seq_len"],
                 kv_layout=kv_layout, force_path=force_path, num_splits=num_splits,
-                waves_per_group=waves_per_group)
+                waves_per_group=waves_per_group, workspace_side=workspace_side)
     plan = ops.mha_plan(ops.make_mha_args(q_d, k_d, v_d, out, ws, **scal))
     ops.mha_decode(q_d, k_d, v_d, out, ws, output_f32=out32, **scal)
     torch.cuda.synchronize()

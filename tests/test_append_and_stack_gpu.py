@@ -441,8 +441,10 @@ def test_attention_block_stack_matches_the_oracle_chain(oracle, dev, mode):
 
 @pytest.mark.parametrize("n_q,ctx,hidden,want_launches,extra", [
     (32, 4096, 2560, 1, {}),      # Qwen3-4B: 32 splits, 248 worker workgroups, rows dealt 3 / 3 / 2 per wavefront
+    (32, 4096, 2560, 1, {"num_splits": 32, "force_path": B.PATH_SPLIT_FUSED}),  # the same plan in both forms: same bits
+    (32, 8192, 2560, 1, {}),
     (32, 3500, 2560, 1, {}),
-    (32, 1500, 2560, 2, {}),      # 16 splits: 480 worker wavefronts of 3 rows are too few for 2560 rows
+    (32, 1500, 2560, 1, {}),      # (the dispatcher would take 16 splits here: the one-launch form asks for 32 itself)
     (16, 700, 1024, 1, {}),       # Qwen3-0.6B head layout
     (64, 5000, 640, 2, {}),       # attention output wider than the fused form takes: two launches, same answer
     (32, 100, 2560, 2, {}),       # single pass: nothing idles, two launches
@@ -450,8 +452,8 @@ def test_attention_block_stack_matches_the_oracle_chain(oracle, dev, mode):
 ])
 def test_fused_output_projection_equals_attention_then_gemv_add(oracle, dev, n_q, ctx, hidden, want_launches, extra):
     """llmi_hip_mha_decode_append_oproj against llmi_hip_mha_decode_append followed by llmi_hip_gemv (add mode) on
-    the same inputs: same attention output and same residual bit for bit, whichever form runs; the attention
-    output also against the oracle. Called three times in a row on one workspace (its per-head counters move on)."""
+    the same inputs: same attention output and same residual bit for bit where both forms run the same plan; the
+    attention output also against the oracle. Called three times in a row on one workspace (its per-head counters move on)."""
     n_kv, d = 8, 128
     rng = np.random.RandomState(ctx + hidden)
     msl, pos, kv_dim, dim = ctx + 2, ctx, n_kv * d, n_q * d
@@ -492,8 +494,17 @@ def test_fused_output_projection_equals_attention_then_gemv_add(oracle, dev, n_q
         launches = ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_b, ws, o_weight=wo_d, residual=res_b, **kw)
         torch.cuda.synchronize()
         assert launches == want_launches
-        assert torch.equal(out_b, out_a), "call %d: attention outputs differ" % call
-        assert torch.equal(res_b, res_a), "call %d: residuals differ" % call
+        # The one-launch form may ask for more splits than the dispatcher would pick on its own (it needs idle
+        # workgroups): the attention output is then the oracle's within the gate instead of the two-call form's bits,
+        # and the residual is, bit for bit, what the GEMV makes of that output.
+        assert_parity(from_dev_bf16(out_b), ref, "call %d: attention inside the one-launch form" % call)
+        res_chk = to_dev(res0, dev)
+        ops.gemv(out_b, wo_d.view(hidden, dim), res_chk, mode=B.GEMV_ADD_BF16)
+        torch.cuda.synchronize()
+        assert torch.equal(res_b, res_chk), "call %d: residuals differ" % call
+        if "num_splits" in extra or launches == 2:
+            assert torch.equal(out_b, out_a), "call %d: attention outputs differ" % call
+            assert torch.equal(res_b, res_a), "call %d: residuals differ" % call
     n = ctypes.c_uint64()
     assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(n)) == 0
 

@@ -5,9 +5,10 @@ import ctypes
 
 import numpy as np
 import pytest
+import torch
 
 from llminfer_amd import _binding as B
-from llminfer_amd import synth
+from llminfer_amd import ops, synth
 
 from helpers import assert_parity, assert_tap_parity, run_hip, run_oracle
 
@@ -307,3 +308,69 @@ def test_random_shapes_against_oracle(oracle, dev, i, kv_mul, n_kv, ctx, slack, 
     position, layer, layout, path, split count and wave count: combinations no hand-written case names."""
     case = synth.make_case(1000 + i, n_q=kv_mul * n_kv, n_kv=n_kv, ctx=ctx, max_seq_len=ctx + slack, layers=layers, layer_id=layer_id)
     _check(oracle, dev, case, kv_layout=layout, force_path=path, num_splits=splits, waves_per_group=waves)
+
+
+def _flip_sides(word):
+    """The measured sides with 1 and 2 exchanged in every region: the layout that puts everything in far memory."""
+    word &= 0xFFFFFFFF
+    out = 0
+    for i in range(16):
+        out |= {1: 2, 2: 1}.get((word >> (2 * i)) & 3, 0) << (2 * i)
+    return out - (1 << 32) if out >> 31 else out
+
+
+@pytest.mark.parametrize("n_q,ctx,splits,offset", [
+    (32, 4096, 0, 0), (32, 1024, 0, 4096), (32, 4097, 32, 8192 + 256), (32, 777, 7, 16), (64, 9000, 0, 0), (16, 3000, 0, 12288),
+    (8, 2000, 16, 0), (40, 5000, 0, 0), (32, 32768, 0, (1 << 20) + 512), (32, 4096, 256, 0),
+])
+def test_workspace_laid_out_by_package_side(oracle, dev, n_q, ctx, splits, offset):
+    """llmi_hip_mha_workspace_side + workspace_side: two homes per row of the fused combine's workspace, each workgroup
+    using the one near its XCD. The result is the plain layout's bit for bit, whichever sides are claimed -- the
+    measured ones, their opposite (everything far), or a made-up word -- and the oracle's; the plan says the layout is in use."""
+    case = synth.make_case(40 + ctx, n_q=n_q, n_kv=8, ctx=ctx)
+    ref = run_oracle(oracle, case)
+    kw = dict(kv_layout=B.KV_LAYOUT_HEAD_MAJOR, force_path=B.PATH_SPLIT_FUSED, num_splits=splits, workspace_offset=offset)
+    plain16, plain32 = run_hip(case, dev, **kw)
+    assert_parity(plain16, ref, "plain layout")
+    ws = torch.empty(ops.workspace_bytes(n_q, 128, ctx + 1) // 4 + offset // 4, dtype=torch.float32, device=dev)[offset // 4:]
+    measured = ops.workspace_side(ws)
+    assert measured == ops.workspace_side(ws)           # the measurement repeats
+    assert any((measured >> (2 * i)) & 3 in (1, 2) for i in range(16))
+    for side in (measured, _flip_sides(measured), 0x66666666, 0x11111111 | (2 << 2)):
+        got16, got32, plan = run_hip(case, dev, want_plan=True, workspace_side=side, **kw)
+        assert plan.workspace_side in (1, 2), "side word %x" % (side & 0xFFFFFFFF)
+        assert np.array_equal(got16, plain16) and np.array_equal(got32, plain32), "side word %x" % (side & 0xFFFFFFFF)
+
+
+def test_workspace_side_falls_back_to_the_plain_layout(oracle, dev):
+    """Where the layout by side does not apply -- unknown sides, a workspace without room for two homes per row, a KV
+    head count that is no multiple of eight, the separate combine kernel, a single pass -- the call runs as before."""
+    case = synth.make_case(77, n_q=32, n_kv=8, ctx=4096)
+    ref = run_oracle(oracle, case)
+    small = 32 * 32 * 528 + 16  # exactly the plain layout's need at 32 splits
+    for kw in (dict(workspace_side=0), dict(workspace_side=1, workspace_bytes=small, num_splits=32),
+               dict(workspace_side=1, force_path=B.PATH_SPLIT, num_splits=32), dict(workspace_side=1, force_path=B.PATH_SINGLE_PASS)):
+        got16, _, plan = run_hip(case, dev, want_plan=True, kv_layout=B.KV_LAYOUT_HEAD_MAJOR, **kw)
+        assert plan.workspace_side == 0
+        assert_parity(got16, ref, str(kw))
+    case = synth.make_case(78, n_q=12, n_kv=4, ctx=3000)
+    got16, _, plan = run_hip(case, dev, want_plan=True, workspace_side=1)
+    assert plan.workspace_side == 0
+    assert_parity(got16, run_oracle(oracle, case), "4 KV heads")
+
+
+def test_workspace_side_argument_checks(dev):
+    ws = torch.empty(1 << 20, dtype=torch.float32, device=dev)
+    side = ctypes.c_int32(-1)
+    f = B.lib().llmi_hip_mha_workspace_side
+    st = torch.cuda.current_stream().cuda_stream
+    assert f(None, 1 << 22, st, ctypes.byref(side)) == B.STATUS["NULL_POINTER"]
+    assert f(ws.data_ptr(), 1 << 22, st, None) == B.STATUS["NULL_POINTER"]
+    assert f(ws.data_ptr() + 4, 1 << 22, st, ctypes.byref(side)) == B.STATUS["ALIGNMENT"]
+    assert f(ws.data_ptr(), 40 << 10, st, ctypes.byref(side)) == B.STATUS["WORKSPACE"]
+    g = torch.cuda.CUDAGraph()
+    s2 = torch.cuda.Stream()
+    with torch.cuda.stream(s2):
+        with torch.cuda.graph(g, stream=s2):
+            assert f(ws.data_ptr(), 1 << 22, s2.cuda_stream, ctypes.byref(side)) == B.STATUS["INVALID_ARG"]  # not under capture
+            torch.zeros(4, device=dev).add_(1)

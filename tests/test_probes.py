@@ -36,16 +36,16 @@ def test_copy_and_handover_reject_bad_arguments():
     assert lib.llmi_hip_probe_copy(None, P, 16, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_copy(P, P, 24, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_copy(P, P + 4, 16, None) == B.STATUS["ALIGNMENT"]
-    assert lib.llmi_hip_probe_handover(0, 2, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_handover(0, 2, 0, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_placement(256, 0, None, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_placement(0, 0, P, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_placement(4097, 0, P, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_placement(256, 0, P + 2, None) == B.STATUS["ALIGNMENT"]
     res = B.ProbeHandoverResult()
-    assert lib.llmi_hip_probe_handover(5, 2, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 16, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 8, 0, P + 16, ctypes.byref(res), None) == B.STATUS["ALIGNMENT"]
+    assert lib.llmi_hip_probe_handover(5, 2, 0, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 0, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 0, 16, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert lib.llmi_hip_probe_handover(0, 2, 3, 8, 0, P + 16, ctypes.byref(res), None) == B.STATUS["ALIGNMENT"]
 
 
 @pytest.fixture(scope="module")
@@ -101,7 +101,7 @@ def test_handover_probe_device_scope_sees_the_store(dev, reader):
     line = torch.zeros(4096 // 4 + 64, dtype=torch.int32, device=dev)
     base = (line.data_ptr() + 255) & ~255
     res = torch.zeros(8, dtype=torch.int32, device=dev)
-    rc = B.lib().llmi_hip_probe_handover(B.PROBE_SC1, B.PROBE_SC1, reader, 1, base, res.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    rc = B.lib().llmi_hip_probe_handover(B.PROBE_SC1, B.PROBE_SC1, 0, reader, 1, base, res.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     seen, polls, ns, xr, xw = (int(x) for x in res[:5].cpu())
