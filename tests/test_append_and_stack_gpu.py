@@ -199,6 +199,19 @@ def test_fused_append_attention(oracle, dev, layout, n_q, n_kv, ctx, path, split
     keep = np.ones(msl, dtype=bool)
     keep[pos] = False
     assert np.array_equal(kc[0, keep], k0[0, keep]) and np.array_equal(vc[0, keep], v0[0, keep])
+    if ctx <= 4096:
+        # the same call with the workspace laid out by package side (measured, then the opposite claim): same bits
+        measured = ops.workspace_side(ws)
+        for side in (measured, 0x55555555 if measured & 2 else -1431655766):
+            k2 = to_dev(synth.to_head_major(k0, n_kv) if hm else k0, dev)
+            v2 = to_dev(synth.to_head_major(v0, n_kv) if hm else v0, dev)
+            out2 = torch.zeros_like(out)
+            ops.mha_decode_append(to_dev(q_raw.reshape(-1), dev), to_dev(k_new.reshape(-1), dev),
+                                  to_dev(v_new.reshape(-1), dev), to_dev(w, dev), sin_d, cos_d, k2, v2, out2, ws,
+                                  layer_id=0, pos=pos, kv_dim=kv_dim, kv_mul=n_q // n_kv, head_num=n_q, head_dim=d,
+                                  max_seq_len=msl, kv_layout=layout, force_path=path, num_splits=splits, workspace_side=side)
+            torch.cuda.synchronize()
+            assert torch.equal(out2, out) and torch.equal(k2, k_d) and torch.equal(v2, v_d), "workspace_side %x" % (side & 0xFFFFFFFF)
 
 
 def test_default_pool_on_device(dev):

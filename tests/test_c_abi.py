@@ -137,6 +137,27 @@ def test_plan_groups_of_eight_query_heads():
         assert p.num_splits == splits and p.rows_per_split == -(-((ctx + 15) // 16) // splits) * 16
 
 
+def test_plan_with_a_measured_workspace_side():
+    """workspace_side set: the fused combine's arrays move to the next 16 KiB boundary and keep two homes per row, if
+    the shape qualifies (a multiple of eight KV heads, one wavefront per query head of a group, at most 128 heads) and
+    the workspace has the room; otherwise the plain layout, without an error."""
+    rc, p = plan(good_args(workspace_side=1, workspace=0x2000))
+    rows = 32 * p.num_splits
+    assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and p.workspace_side == 1
+    assert p.workspace_needed == (0x4000 - 0x2000) + 2 * -(-rows // 16) * 8192 + 2 * -(-rows // 512) * 8192 + 16
+    rc, p0 = plan(good_args(workspace_side=0, workspace=0x2000))
+    assert rc == 0 and p0.workspace_side == 0 and p0.num_splits == p.num_splits and p0.workspace_needed == rows * 528 + 16
+    assert B.lib().llmi_hip_mha_workspace_bytes(32, 128, 4096) >= p.workspace_needed + 8192 + 32 * 4
+    for over in (dict(workspace_bytes=p.workspace_needed - 1),                 # no room for two homes
+                 dict(kv_mul=8, head_num=32, kv_dim=512),                       # 4 KV heads
+                 dict(waves_per_group=2),                                       # fewer wavefronts than heads in a group
+                 dict(force_path=B.PATH_SPLIT, num_splits=8), dict(pos=100)):   # separate combine kernel, single pass
+        rc, q = plan(good_args(workspace_side=1, workspace=0x2000, **over))
+        assert rc == 0 and q.workspace_side == 0, over
+    rc, p = plan(good_args(workspace_side=-1431655766, workspace=0x4000))  # (0xAAAAAAAA as int32: any word is taken)
+    assert rc == 0 and p.workspace_side == 1 and p.workspace_needed == 2 * -(-rows // 16) * 8192 + 2 * -(-rows // 512) * 8192 + 16
+
+
 def test_plan_honours_requests_and_clamps_to_the_workspace():
     rc, p = plan(good_args(force_path=B.PATH_SPLIT, num_splits=16))
     assert rc == 0 and p.path == B.PATH_SPLIT and p.num_splits == 16 and p.rows_per_split == 256
@@ -251,11 +272,12 @@ def test_plan_invariants_over_random_arguments():
     @hyp.settings(max_examples=600, deadline=None, derandomize=True)
     @hyp.given(kv_mul=st.integers(1, 16), n_kv=st.sampled_from([1, 2, 4, 8, 16]), ctx=st.integers(1, 140000),
                slack=st.integers(0, 64), force_path=st.integers(0, 3), num_splits=st.sampled_from([0, 0, 0, 1, 2, 3, 7, 32, 200, 256]),
-               waves=st.sampled_from([0, 0, 1, 2, 4, 8]), ws_kib=st.sampled_from([0, 1, 64, 4096, 1 << 17]))
-    def check(kv_mul, n_kv, ctx, slack, force_path, num_splits, waves, ws_kib):
+               waves=st.sampled_from([0, 0, 1, 2, 4, 8]), ws_kib=st.sampled_from([0, 1, 64, 4096, 1 << 17]),
+               side=st.sampled_from([0, 0, 1, 2, 0x66, -1]))
+    def check(kv_mul, n_kv, ctx, slack, force_path, num_splits, waves, ws_kib, side):
         a = good_args(pos=ctx - 1, max_seq_len=ctx + slack, kv_mul=kv_mul, kv_dim=128 * n_kv, head_num=kv_mul * n_kv,
                       force_path=force_path, num_splits=num_splits, waves_per_group=waves,
-                      workspace=0x2000 if ws_kib else 0, workspace_bytes=ws_kib << 10)
+                      workspace=0x2000 if ws_kib else 0, workspace_bytes=ws_kib << 10, workspace_side=side)
         rc, p = plan(a)
         if rc != 0:
             assert rc in (B.STATUS["WORKSPACE"], B.STATUS["INVALID_ARG"])
@@ -265,6 +287,7 @@ def test_plan_invariants_over_random_arguments():
         assert p.rows_per_split % 16 == 0 and p.rows_per_split == -(-tiles // p.num_splits) * 16
         assert (p.num_splits == 1) == (p.path == B.PATH_SINGLE_PASS)
         assert p.workspace_needed <= (ws_kib << 10) and (p.num_splits == 1) == (p.workspace_needed == 0)
+        assert p.workspace_side in (0, 1) and (p.workspace_side == 0 or (side != 0 and n_kv % 8 == 0 and p.path == B.PATH_SPLIT_FUSED))
         assert p.group_pad in (1, 2, 4, 8, 16) and kv_mul <= p.group_pad < 2 * kv_mul
         assert p.waves_per_group in (1, 2, 4, 8) and p.group_pad * p.waves_per_group <= 64
         if waves:

@@ -37,6 +37,8 @@ def test_copy_and_handover_reject_bad_arguments():
     assert lib.llmi_hip_probe_copy(P, P, 24, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_copy(P, P + 4, 16, None) == B.STATUS["ALIGNMENT"]
     assert lib.llmi_hip_probe_handover(0, 2, 0, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_block_pingpong(None, P, P, None) == B.STATUS["NULL_POINTER"]
+    assert lib.llmi_hip_probe_block_pingpong(P, P + 128, P, None) == B.STATUS["ALIGNMENT"]
     assert lib.llmi_hip_probe_placement(256, 0, None, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_placement(0, 0, P, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_placement(4097, 0, P, None) == B.STATUS["INVALID_ARG"]
@@ -124,3 +126,24 @@ def test_placement_probe_names_a_cu_for_every_workgroup(dev, exclusive):
     cus = {(int(x), (int(h) >> 8) & 0xFF) for x, h in a}
     assert len(cus) >= 128
     assert len(set(int(x) for x in a[:, 0])) >= 1
+
+
+@pytest.mark.gpu
+def test_pingpong_probe_times_both_blocks_from_every_xcd(dev):
+    """Eight pairs of workgroups, each pair on one XCD, hand 64 numbers to and fro through two neighbouring 8 KiB blocks:
+    every number arrives, the pairs cover both sides of the package, the times are a few hundred ns per hand-over, and
+    the two sides disagree about which block is nearer (what llmi_hip_mha_workspace_side reads off)."""
+    import torch
+    buf = torch.zeros((64 << 10) // 4, dtype=torch.int32, device=dev)
+    base = (buf.data_ptr() + 16383) & ~16383
+    out = torch.zeros(64, dtype=torch.int32, device=dev)
+    assert B.lib().llmi_hip_probe_block_pingpong(base, base + 8192, out.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    r = out.cpu().numpy().astype(np.int64).reshape(8, 8)
+    assert np.all(r[:, 3] == 1)                                   # nothing lost
+    assert np.all(r[:, 0] == r[:, 5]) and np.all(r[:, 0] < 8)     # a pair shares an XCD
+    assert {int(x) >> 2 for x in r[:, 0]} == {0, 1}               # both sides of the package
+    per_handover_ns = r[:, 1:3] * 10 / 64
+    assert np.all(per_handover_ns > 100) and np.all(per_handover_ns < 5000)
+    d = [np.mean((r[:, 1] - r[:, 2])[(r[:, 0] >> 2) == s]) for s in (0, 1)]
+    assert d[0] * d[1] < 0
