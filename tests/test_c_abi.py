@@ -300,3 +300,16 @@ def test_plan_invariants_over_random_arguments():
             assert p.path == force_path
 
     check()
+
+
+def test_build_rejects_kernels_with_a_private_segment():
+    """The build reads the compiler's resource-usage remarks and refuses a kernel that was given scratch memory."""
+    from llminfer_amd import build
+    remarks = "\n".join([
+        "a.hip:1:1: remark: Function Name: kern_a [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:9:1: remark: Function Name: kern_b [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:9:1: remark:     VGPRs: 14 [-Rpass-analysis=kernel-resource-usage]",
+        "a.hip:9:1: remark:     ScratchSize [bytes/lane]: 48 [-Rpass-analysis=kernel-resource-usage]"])
+    assert build.kernels_using_scratch(remarks) == ["kern_b"]
+    assert build.kernels_using_scratch("") == []
