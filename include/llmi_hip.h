@@ -338,6 +338,14 @@ int llmi_hip_abi_version(void);
  * after the call; returns the previous limit. 0 makes every fused launch give up at once: the way to
  * exercise the failure path in a test. */
 int32_t llmi_hip_set_poll_limit(int32_t polls);
+/* No counterpart in the reference; a testing aid like the one above. With the workspace laid out by package side a
+ * split keeps its partial results and record in the home near its own XCD, and the workgroup that merges finds them in
+ * the home near itself because both run on one XCD. `mode` 1 makes every split but the merging one use the OTHER home,
+ * mode 2 every second split: what a launch would look like whose workgroups were not dealt to the XCDs as expected.
+ * The merging workgroup must then find the records by its fall-back (both homes, after 16 rounds of polls) and read
+ * every split's partial results from the right home: same result, a few microseconds later. 0 (the default) switches
+ * it off. Applies to launches enqueued after the call; returns the previous mode. */
+int32_t llmi_hip_set_test_far_home(int32_t mode);
 /* No counterpart in the reference. How many of those bounded waits have given up on the current device since
  * the library was loaded (one count per query head and call; the NaN outputs are the other sign). Reads a
  * device counter with a synchronous copy: it waits for work already enqueued on the device and must not be

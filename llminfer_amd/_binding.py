@@ -126,6 +126,7 @@ SYMBOLS = {
     "llmi_hip_memset_zero": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, c_i32]),
     "llmi_hip_abi_version": (ctypes.c_int, []),
     "llmi_hip_set_poll_limit": (c_i32, [c_i32]),
+    "llmi_hip_set_test_far_home": (c_i32, [c_i32]),
     "llmi_hip_poll_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint64)]),
     # include/llmi_hip_probes.h
     "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),

@@ -66,6 +66,8 @@ unsigned long long next_epoch() {
 // Default: far beyond any real kernel time (seconds), yet finite.
 static std::atomic<int> g_poll_limit{1 << 22};
 int poll_limit() { return g_poll_limit.load(std::memory_order_relaxed); }
+static std::atomic<int> g_test_far_home{0};
+int test_far_home() { return g_test_far_home.load(std::memory_order_relaxed); }
 
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
 
@@ -535,6 +537,10 @@ int llmi_hip_qkv_gemv(const llmi_qkv_gemv_args* a) {
 }
 
 int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }
+
+int32_t llmi_hip_set_test_far_home(int32_t mode) {
+    return llmi::g_test_far_home.exchange(mode < 0 || mode > 2 ? 0 : mode, std::memory_order_relaxed);
+}
 
 int32_t llmi_hip_set_poll_limit(int32_t polls) {
     return llmi::g_poll_limit.exchange(polls < 0 ? 0 : polls, std::memory_order_relaxed);

@@ -64,6 +64,9 @@ inline size_t side_pad(const void* workspace) { return (size_t)(-reinterpret_cas
 int read_poll_timeouts(unsigned long long* count);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.
 int poll_limit();
+// Testing aid (llmi_hip_set_test_far_home): 1 = every split but the merging one, 2 = every second split stores into
+// the home of the other side of the package.
+int test_far_home();
 
 // `append` non-null: the fused QK-Norm + RoPE + K/V append variant.
 // `oproj` non-null (with `append`): the attention launch also computes the output projection + residual add.

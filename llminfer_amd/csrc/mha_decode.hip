@@ -256,6 +256,7 @@ struct KernelArgs {
     // partial outputs / records; XCDs 4-7 use the other one.
     bool by_side;
     unsigned long long ppar[2], rpar[2];
+    int32_t far_home;  // testing aid: 1 = every split but the merging one, 2 = every second one uses the other side's home
 };
 
 // What the attention part of an OPROJ kernel hands to the projection part.
@@ -274,7 +275,7 @@ struct OprojState {
 // the combiner polls the records' home near itself and reads a split's partial outputs from the home that goes with
 // the one it found the record in. With the KV head in blockIdx.x and a KV head count that is a multiple of eight, all
 // workgroups of a KV head run on one XCD (they are dealt to the XCDs in turn), so they agree on the home and
-// everything they hand over travels through near memory. Nothing relies on that placement for its result: after 64
+// everything they hand over travels through near memory. Nothing relies on that placement for its result: after 16
 // rounds of polls the combiner also looks into the other home for the records it is still missing, so a split that
 // ran on the other side is found later, not never. Which block of a pair is near which side is what
 // llmi_hip_mha_workspace_side measures, per 2 MiB region; the launcher turns it into one bit per head and array.
@@ -773,6 +774,8 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
 
     const bool fused = a.records != nullptr && n_active > 1;
     const int my_xs = package_side(a);  // wave-uniform: the side of the package this workgroup runs on
+    // (testing aid: pretend this split ran on the other side; never the merging one, whose own rows it reads itself)
+    const int store_xs = my_xs ^ (int)(a.by_side && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     if constexpr (OPROJ) proj.worker = split != n_active - 1;
     // One thread per (head, 16-byte column): weights e^(m_w - M) of the waves, weighted sum.
     const int n_units = a.group * (kHeadDim / 4);
@@ -811,7 +814,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         } else {
             const int64_t S = a.num_splits;
             const WsHead wh = ws_head(a, hq);
-            const int64_t po = (fused ? (int64_t)ws_row<4>(wh, split, my_xs) : (int64_t)hq * S + split) * kHeadDim + c4 * 4;  // element offset in the workspace
+            const int64_t po = (fused ? (int64_t)ws_row<4>(wh, split, store_xs) : (int64_t)hq * S + split) * kHeadDim + c4 * 4;  // element offset in the workspace
             if (fused) {
                 // Device-coherent store (cache policy sc1): it goes past this XCD's L2, so the
                 // workgroup (possibly on another XCD) that does the combine can read it without
@@ -824,7 +827,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                     // workgroup barrier is needed.
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     if (c4 == 0) {
-                        unsigned long long* rec = a.records + (int64_t)ws_row<9>(wh, split, my_xs) * 2;
+                        unsigned long long* rec = a.records + (int64_t)ws_row<9>(wh, split, store_xs) * 2;
                         const unsigned long long tag = a.tag;
                         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, mx);
                         const unsigned long long l_bits = __builtin_bit_cast(uint32_t, lsum);
@@ -922,8 +925,8 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             }
             return __all(ok);
         };
-        // The first rounds poll the near home only (a few tens of microseconds: far beyond the spread of the splits).
-        constexpr int kNearRounds = 64;
+        // The first rounds poll the near home only (some ten microseconds: far beyond the spread of the splits).
+        constexpr int kNearRounds = 16;
         const int near_rounds = wh.by_side ? min(a.max_polls, kNearRounds) : a.max_polls;
         bool all_in = false;
         for (int spin = 0; spin < near_rounds && !all_in; ++spin) {
@@ -1434,6 +1437,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
             if (pad + fw.bytes() > args.workspace_bytes) return LLMI_ERR_WORKSPACE;  // (the plan was made for this workspace)
             base += pad;
             ka.by_side = true;
+            ka.far_home = test_far_home();
             ka.ws = reinterpret_cast<float*>(base);
             // One rule per head, taken from the region its first row lies in (a head whose rows straddle a region
             // boundary has some of them in far memory, nothing else): two bits per 2 MiB region in workspace_side,

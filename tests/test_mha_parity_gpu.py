@@ -374,3 +374,31 @@ def test_workspace_side_argument_checks(dev):
         with torch.cuda.graph(g, stream=s2):
             assert f(ws.data_ptr(), 1 << 22, s2.cuda_stream, ctypes.byref(side)) == B.STATUS["INVALID_ARG"]  # not under capture
             torch.zeros(4, device=dev).add_(1)
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("n_q,ctx,splits", [(32, 4096, 0), (32, 5000, 32), (64, 9000, 0), (32, 20000, 100), (16, 700, 5)])
+def test_splits_that_used_the_other_home_are_still_found(oracle, dev, mode, n_q, ctx, splits):
+    """llmi_hip_set_test_far_home: every split but the merging one (mode 1), or every second split (mode 2), keeps its
+    partial results and record in the home of the OTHER side of the package, as if the workgroups of a KV head had not
+    shared an XCD. The merging workgroup finds nothing (or half) in the home it polls, falls back to both homes after 16
+    rounds and reads every split's rows from where its record was: the bits of the undisturbed call, no give-up counted,
+    also on the next call and with the opposite sides claimed."""
+    case = synth.make_case(60 + ctx, n_q=n_q, n_kv=8, ctx=ctx)
+    kw = dict(kv_layout=B.KV_LAYOUT_HEAD_MAJOR, force_path=B.PATH_SPLIT_FUSED, num_splits=splits)
+    want16, want32, plan = run_hip(case, dev, want_plan=True, workspace_side="measure", **kw)
+    assert plan.workspace_side == 1
+    assert_parity(want16, run_oracle(oracle, case), "undisturbed")
+    timeouts = ctypes.c_uint64()
+    assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(timeouts)) == 0
+    before = timeouts.value
+    assert B.lib().llmi_hip_set_test_far_home(mode) == 0
+    try:
+        for side in ("measure", 0x55555555, -1431655766):
+            got16, got32 = run_hip(case, dev, workspace_side=side, **kw)
+            assert np.array_equal(got16, want16) and np.array_equal(got32, want32), "mode %d sides %s" % (mode, side)
+    finally:
+        assert B.lib().llmi_hip_set_test_far_home(0) == mode
+    again16, again32 = run_hip(case, dev, workspace_side="measure", **kw)
+    assert np.array_equal(again16, want16) and np.array_equal(again32, want32)
+    assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(timeouts)) == 0 and timeouts.value == before
