@@ -9,6 +9,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 #include "llmi_hip.h"
@@ -257,19 +258,23 @@ int llmi_hip_mha_decode_static(const llmi_mha_args* args) {
         if (int rc = record_hip_error(hipGetDevice(&dev), "hipGetDevice")) return rc;
         int32_t sides = 0;
         if (dev >= 0 && dev < kMaxDevices) {
-            if (measured[dev].load(std::memory_order_acquire)) {
-                sides = sides_of[dev].load(std::memory_order_relaxed);
-            } else {
+            if (!measured[dev].load(std::memory_order_acquire)) {
+                static std::mutex measuring;  // (two first calls at once would measure through the same lines)
+                std::lock_guard<std::mutex> lock(measuring);
                 hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
                 hipStream_t s = static_cast<hipStream_t>(a.stream);
-                if (hipStreamIsCapturing(s, &cs) == hipSuccess && cs == hipStreamCaptureStatusNone) {
-                    if (int rc = measure_workspace_side(ptr, bytes, s, &sides)) return rc;
-                    sides_of[dev].store(sides, std::memory_order_relaxed);
+                if (measured[dev].load(std::memory_order_acquire)) {
+                    // (another thread got there first)
+                } else if (hipStreamIsCapturing(s, &cs) == hipSuccess && cs == hipStreamCaptureStatusNone) {
+                    int32_t found = 0;
+                    if (int rc = measure_workspace_side(ptr, bytes, s, &found)) return rc;
+                    sides_of[dev].store(found, std::memory_order_relaxed);
                     measured[dev].store(1, std::memory_order_release);
                 } else {
-                    (void)hipGetLastError();  // (this call only: the plain layout)
+                    (void)hipGetLastError();  // (under capture: this call keeps the plain layout)
                 }
             }
+            if (measured[dev].load(std::memory_order_acquire)) sides = sides_of[dev].load(std::memory_order_relaxed);
         }
         a.workspace_side = sides;
         if (a.workspace_side != args->workspace_side)
