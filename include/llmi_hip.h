@@ -27,6 +27,10 @@
  *                                 code/source/op/kernel/cuda/rope_kernel.cu:23-46
  *   llmi_hip_kv_restride          (new) converts a position-major cache
  *                                 (qwen3_fused.cpp:488-491) to the head-major layout
+ *   llmi_hip_mha_workspace_side   (new) measures, once per KVSplitOutput allocation
+ *                                 (qwen3_fused.cpp:502-503), which of its 8 KiB blocks lie near
+ *                                 which side of the GPU package; llmi_mha_args.workspace_side
+ *   llmi_hip_mha_decode_static    (new) llmi_hip_mha_decode without a caller's workspace
  *   llmi_pool_* / llmi_hip_pool_* base::CUDADeviceAllocator::allocate / release
  *                                 code/source/base/alloc_cu.cpp:7-119
  *   llmi_hip_memcpy / memset_zero base::DeviceAllocator::memcpy / memset_zero
