@@ -198,11 +198,12 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
                                                           : per_split_plain * (size_t)num_splits;
     // The workspace laid out by package side: where every split of a KV head and its combiner run on one XCD (the KV
     // head is the fastest grid index and the head count a multiple of the eight XCDs), where one wavefront merges
-    // a head (the shared read-back of larger groups keeps the plain layout), and where the workspace has room
+    // a head (the shared read-back of larger groups keeps the plain layout), with the wave count the dispatcher picks
+    // itself (the only ones the kernel is built for in this layout), and where the workspace has room
     // for two homes per row, rounded to whole 8 KiB blocks, behind the way to the next 16 KiB boundary. Otherwise the
     // plain layout, silently: the side only ever changes the time.
     if (path == LLMI_PATH_SPLIT_FUSED && num_splits > 1 && a->workspace_side != 0 && n_kv % 8 == 0 && a->kv_mul <= waves &&
-        a->head_num <= 128) {
+        a->head_num <= 128 && by_side_variant(group_pad, waves)) {
         const size_t need = side_pad(a->workspace) + fused_workspace(a->head_num, a->head_dim, num_splits, true).bytes();
         if (a->workspace_bytes >= need) {
             p->workspace_side = 1;

@@ -60,6 +60,9 @@ int measure_workspace_side(void* workspace, size_t bytes, hipStream_t stream, in
 // Bytes from a workspace's start to the by-side layout: the next 16 KiB boundary (a row's two homes are the two
 // 8 KiB blocks of an aligned pair, so that both lie in one region).
 inline size_t side_pad(const void* workspace) { return (size_t)(-reinterpret_cast<intptr_t>(workspace)) & (2 * kSideBlock - 1); }
+// The kernel is built for the by-side layout with the wave counts the dispatcher picks itself: four wavefronts per
+// workgroup, eight for (padded) groups of 8 query heads. Other wave counts keep the plain layout.
+constexpr bool by_side_variant(int group_pad, int waves) { return group_pad <= 8 && waves == (group_pad == 8 ? 8 : 4); }
 // Waits of the fused combine that gave up since the library was loaded (device counter of the current device).
 int read_poll_timeouts(unsigned long long* count);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.

@@ -284,9 +284,11 @@ struct WsHead {
     bool by_side;
     int ppar, rpar;  // partials / records: which block of a pair (address bit 13) side 0 of the package uses for this head
 };
+// BYSIDE is a kernel's compile-time choice: the plain layout's instantiations carry none of the other's code.
+template <bool BYSIDE>
 __device__ __forceinline__ WsHead ws_head(const KernelArgs& a, int hq) {
-    WsHead w{hq * a.num_splits, a.by_side, 0, 0};
-    if (a.by_side) {
+    WsHead w{hq * a.num_splits, BYSIDE, 0, 0};
+    if constexpr (BYSIDE) {
         w.ppar = (int)(((hq < 64 ? a.ppar[0] : a.ppar[1]) >> (hq & 63)) & 1ull);
         w.rpar = (int)(((hq < 64 ? a.rpar[0] : a.rpar[1]) >> (hq & 63)) & 1ull);
     }
@@ -303,8 +305,9 @@ __device__ __forceinline__ int ws_row(const WsHead& w, int sp, int xs) {
 }
 constexpr uint32_t kSideBlockBytes = 8192u;
 // Side of the package this workgroup's XCD is on (0 in the plain layout).
-__device__ __forceinline__ int package_side(const KernelArgs& a) {
-    if (!a.by_side) return 0;
+template <bool BYSIDE>
+__device__ __forceinline__ int package_side() {
+    if constexpr (!BYSIDE) return 0;
     uint32_t xcc;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
     return (int)((xcc >> 2) & 1u);
@@ -363,7 +366,7 @@ __device__ __forceinline__ void norm_rope_rows_lds(char* rows, const char* w, co
 template <int G, int NW>
 constexpr int kWavesPerEu = (G >= 16 && NW != 2) ? 1 : LLMI_MIN_WAVES_PER_EU;
 
-template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER, bool OPROJ>
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER, bool OPROJ, bool BYSIDE>
 __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState& proj) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
@@ -773,13 +776,13 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     __syncthreads();
 
     const bool fused = a.records != nullptr && n_active > 1;
-    const int my_xs = package_side(a);  // wave-uniform: the side of the package this workgroup runs on
+    const int my_xs = package_side<BYSIDE>();  // wave-uniform: the side of the package this workgroup runs on
     // (testing aid: pretend this split ran on the other side; never the merging one, whose own rows it reads itself)
-    const int store_xs = my_xs ^ (int)(a.by_side && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
+    const int store_xs = my_xs ^ (int)(BYSIDE && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     if constexpr (OPROJ) proj.worker = split != n_active - 1;
     // One thread per (head, 16-byte column): weights e^(m_w - M) of the waves, weighted sum.
     const int n_units = a.group * (kHeadDim / 4);
-    const int64_t part_rows = a.by_side ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
+    const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
     const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         a.ws, 0, (int)(part_rows * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
     for (int u = threadIdx.x; u < n_units; u += NW * 64) {
@@ -813,7 +816,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             }
         } else {
             const int64_t S = a.num_splits;
-            const WsHead wh = ws_head(a, hq);
+            const WsHead wh = ws_head<BYSIDE>(a, hq);
             const int64_t po = (fused ? (int64_t)ws_row<4>(wh, split, store_xs) : (int64_t)hq * S + split) * kHeadDim + c4 * 4;  // element offset in the workspace
             if (fused) {
                 // Device-coherent store (cache policy sc1): it goes past this XCD's L2, so the
@@ -886,7 +889,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         bool ok = false;
         // Bounded wait: every wave leaves this loop even if a record never shows up
         // (the result is then poisoned below instead of hanging the GPU).
-        const WsHead wh = ws_head(a, kvh * a.group + h);
+        const WsHead wh = ws_head<BYSIDE>(a, kvh * a.group + h);
         const unsigned long long* rec_near[kSlots];
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) rec_near[j] = a.records + (int64_t)ws_row<9>(wh, min(lane + 64 * j, SA - 1), my_xs) * 2;
@@ -927,15 +930,17 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         };
         // The first rounds poll the near home only (some ten microseconds: far beyond the spread of the splits).
         constexpr int kNearRounds = 16;
-        const int near_rounds = wh.by_side ? min(a.max_polls, kNearRounds) : a.max_polls;
+        const int near_rounds = BYSIDE ? min(a.max_polls, kNearRounds) : a.max_polls;
         bool all_in = false;
         for (int spin = 0; spin < near_rounds && !all_in; ++spin) {
             all_in = poll_round(std::false_type{});
             if (!all_in) __builtin_amdgcn_s_sleep(2);
         }
-        for (int spin = near_rounds; spin < a.max_polls && !all_in; ++spin) {
-            all_in = poll_round(std::true_type{});
-            if (!all_in) __builtin_amdgcn_s_sleep(2);
+        if constexpr (BYSIDE) {
+            for (int spin = near_rounds; spin < a.max_polls && !all_in; ++spin) {
+                all_in = poll_round(std::true_type{});
+                if (!all_in) __builtin_amdgcn_s_sleep(2);
+            }
         }
         const bool arrived = __all(ok);
         // A give-up is counted where the host can read it (llmi_hip_poll_timeouts).
@@ -946,7 +951,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     // of s_w, the denominator sum l_s * weight; the records are zeroed for the next use.
     auto make_weights = [&](int h, auto slots, const float* m_reg, const float* l_reg, const bool* home) -> float {
         constexpr int kSlots = decltype(slots)::value;
-        const WsHead wh = ws_head(a, kvh * a.group + h);
+        const WsHead wh = ws_head<BYSIDE>(a, kvh * a.group + h);
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < kSlots; ++j) mx = fmaxf(mx, m_reg[j]);
@@ -996,12 +1001,12 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         const int part = lane >> 5;
         const int hq = kvh * a.group + h;
         const float* w = s_w + h * kMaxSplits;
-        const WsHead wh = ws_head(a, hq);
+        const WsHead wh = ws_head<BYSIDE>(a, hq);
         // Byte offset of split sp's partial row, in both layouts with the same few instructions: plain, it is
         // B = row * 512; by side, the row's pair of 8 KiB blocks starts at twice B's block start and the home adds 8 KiB
         // or not: B + (B & block_mask) + home, with block_mask = 0 and home = 0 in the plain layout.
         const uint32_t row0_bytes = (uint32_t)wh.rbase * (kHeadDim * 4u);
-        const uint32_t block_mask = wh.by_side ? ~(uint32_t)(kSideBlockBytes - 1) : 0u;
+        const uint32_t block_mask = BYSIDE ? ~(uint32_t)(kSideBlockBytes - 1) : 0u;
         const uint32_t lane_bytes = (uint32_t)c4 * 16u;
         auto load_partial = [&](int sp, uint32_t home_bytes) {
             const int spc = min(sp, SA - 1);  // in range; the weight drops the repeat
@@ -1021,8 +1026,8 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             bool other = false;
 #pragma unroll
             for (int j = 0; j < kSlots; ++j) other = other || home[j] != (my_xs != 0);
-            const bool mixed = wh.by_side && __any(other);
-            const uint32_t near_bytes = wh.by_side ? (uint32_t)(wh.ppar ^ my_xs) * kSideBlockBytes : 0u;
+            const bool mixed = BYSIDE && __any(other);
+            const uint32_t near_bytes = BYSIDE ? (uint32_t)(wh.ppar ^ my_xs) * kSideBlockBytes : 0u;
             float den = 0.0f;
             // The read-back, once for the usual case (every split in this side's home: one constant, nothing between the
             // loads) and once for the other one: two copies of the code rather than a test in front of every load.
@@ -1063,7 +1068,9 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 }
                 return sum;
             };
-            f32x4 acc = mixed ? gather(std::true_type{}) : gather(std::false_type{});
+            f32x4 acc;
+            if constexpr (BYSIDE) acc = mixed ? gather(std::true_type{}) : gather(std::false_type{});
+            else acc = gather(std::false_type{});
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = halves_sum(acc[e]);
             if (part == 0) {
@@ -1191,10 +1198,10 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     }
 }
 
-template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false>
+template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER = false, bool BYSIDE = false>
 __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kernel(KernelArgs a) {
     OprojState unused;
-    mha_decode_body<G, NW, NSTAGE, APPEND, DYN, STAGGER, false>(a, unused);
+    mha_decode_body<G, NW, NSTAGE, APPEND, DYN, STAGGER, false, BYSIDE>(a, unused);
 }
 
 // The attention launch with the layer's output projection and residual add behind it, in the same launch
@@ -1205,10 +1212,10 @@ __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_decode_kern
 // attention output (ordinary loads: see below) and finishes its rows: dot products, residual add, one
 // rounding. The weights stream while HBM would otherwise sit idle behind the attention's hand-over.
 // Needs every workgroup of the grid resident at once (the launcher checks the grid against the CU count).
-template <int G, int NW, int NSTAGE>
+template <int G, int NW, int NSTAGE, bool BYSIDE>
 __global__ __launch_bounds__(NW * 64, (kWavesPerEu<G, NW>)) void mha_oproj_kernel(KernelArgs a) {
     OprojState proj;
-    mha_decode_body<G, NW, NSTAGE, true, false, false, true>(a, proj);
+    mha_decode_body<G, NW, NSTAGE, true, false, false, true, BYSIDE>(a, proj);
     if (!proj.worker) return;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1338,12 +1345,31 @@ __global__ __launch_bounds__(kHeadDim) void mha_combine_kernel(const float* __re
 #define LLMI_RING_LIMIT 65536
 #endif
 
+// The layout by package side has instantiations for the wave counts the dispatcher picks itself; the planner asks
+// for it nowhere else (by_side_variant).
+template <int G, int NW>
+constexpr bool kHasBySide = by_side_variant(G, NW);
+
 template <int G, int NW>
 void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stream) {
     // NW * NSTAGE * 8 KiB of ring must fit the LDS budget of one workgroup.
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
     dim3 grid(n_kv, ka.num_splits);
     const bool dyn = ka.pos_dev != nullptr;  // position read at run time: its own instantiation, the static one pays nothing
+    if constexpr (kHasBySide<G, NW>) {
+        if (ka.by_side) {
+            if (append) {
+                if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+            } else {
+                if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else if (ka.stagger)
+                    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+            }
+            return;
+        }
+    }
     if (append) {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
@@ -1371,7 +1397,13 @@ bool launch_decode_nw(const KernelArgs& ka, int n_kv, int nw, bool append, hipSt
 template <int G, int NW>
 void launch_oproj(const KernelArgs& ka, int n_kv, hipStream_t stream) {
     constexpr int kStages = (NW * LLMI_STAGES * 8192 <= LLMI_RING_LIMIT) ? LLMI_STAGES : LLMI_RING_LIMIT / (NW * 8192);
-    hipLaunchKernelGGL((mha_oproj_kernel<G, NW, kStages>), dim3(n_kv, ka.num_splits), dim3(NW * 64), 0, stream, ka);
+    if constexpr (kHasBySide<G, NW>) {
+        if (ka.by_side) {
+            hipLaunchKernelGGL((mha_oproj_kernel<G, NW, kStages, true>), dim3(n_kv, ka.num_splits), dim3(NW * 64), 0, stream, ka);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((mha_oproj_kernel<G, NW, kStages, false>), dim3(n_kv, ka.num_splits), dim3(NW * 64), 0, stream, ka);
 }
 
 }  // namespace
@@ -1429,7 +1461,7 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
     if (plan.path == LLMI_PATH_SPLIT_FUSED) {
         // Arrival records sit behind the partial outputs in the workspace; laid out by package side, both arrays
         // start on an 8 KiB boundary.
-        const bool by_side = plan.workspace_side != 0;
+        const bool by_side = plan.workspace_side != 0 && by_side_variant(plan.group_pad, plan.waves_per_group);
         const FusedWorkspace fw = fused_workspace(args.head_num, args.head_dim, plan.num_splits, by_side);
         char* base = static_cast<char*>(args.workspace);
         if (by_side) {

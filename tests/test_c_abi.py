@@ -139,8 +139,9 @@ def test_plan_groups_of_eight_query_heads():
 
 def test_plan_with_a_measured_workspace_side():
     """workspace_side set: the fused combine's arrays move to the next 16 KiB boundary and keep two homes per row, if
-    the shape qualifies (a multiple of eight KV heads, one wavefront per query head of a group, at most 128 heads) and
-    the workspace has the room; otherwise the plain layout, without an error."""
+    the shape qualifies (a multiple of eight KV heads, at most 128 heads, groups of at most 8 query heads with the
+    wave count the dispatcher picks itself: the kernel is built for the layout with those) and the workspace has the
+    room; otherwise the plain layout, without an error."""
     rc, p = plan(good_args(workspace_side=1, workspace=0x2000))
     rows = 32 * p.num_splits
     assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and p.workspace_side == 1
@@ -150,12 +151,17 @@ def test_plan_with_a_measured_workspace_side():
     assert B.lib().llmi_hip_mha_workspace_bytes(32, 128, 4096) >= p.workspace_needed + 8192 + 32 * 4
     for over in (dict(workspace_bytes=p.workspace_needed - 1),                 # no room for two homes
                  dict(kv_mul=8, head_num=32, kv_dim=512),                       # 4 KV heads
-                 dict(waves_per_group=2),                                       # fewer wavefronts than heads in a group
+                 dict(waves_per_group=2), dict(waves_per_group=8),              # not the dispatcher's own wave count
+                 dict(kv_mul=16, head_num=128, kv_dim=1024),                    # groups of 16 query heads
                  dict(force_path=B.PATH_SPLIT, num_splits=8), dict(pos=100)):   # separate combine kernel, single pass
         rc, q = plan(good_args(workspace_side=1, workspace=0x2000, **over))
         assert rc == 0 and q.workspace_side == 0, over
     rc, p = plan(good_args(workspace_side=-1431655766, workspace=0x4000))  # (0xAAAAAAAA as int32: any word is taken)
     assert rc == 0 and p.workspace_side == 1 and p.workspace_needed == 2 * -(-rows // 16) * 8192 + 2 * -(-rows // 512) * 8192 + 16
+    rc, p = plan(good_args(workspace_side=1, workspace=0x2000, waves_per_group=4))  # the dispatcher's own count, spelled out
+    assert rc == 0 and p.workspace_side == 1
+    rc, p = plan(good_args(workspace_side=1, workspace=0x2000, kv_mul=8, head_num=64, kv_dim=1024, workspace_bytes=8 << 20))
+    assert rc == 0 and p.workspace_side == 1 and p.waves_per_group == 8
 
 
 def test_plan_honours_requests_and_clamps_to_the_workspace():
@@ -287,7 +293,8 @@ def test_plan_invariants_over_random_arguments():
         assert p.rows_per_split % 16 == 0 and p.rows_per_split == -(-tiles // p.num_splits) * 16
         assert (p.num_splits == 1) == (p.path == B.PATH_SINGLE_PASS)
         assert p.workspace_needed <= (ws_kib << 10) and (p.num_splits == 1) == (p.workspace_needed == 0)
-        assert p.workspace_side in (0, 1) and (p.workspace_side == 0 or (side != 0 and n_kv % 8 == 0 and p.path == B.PATH_SPLIT_FUSED))
+        assert p.workspace_side in (0, 1) and (p.workspace_side == 0 or (side != 0 and n_kv % 8 == 0 and p.path == B.PATH_SPLIT_FUSED
+                                                                 and p.waves_per_group == (8 if p.group_pad == 8 else 4)))
         assert p.group_pad in (1, 2, 4, 8, 16) and kv_mul <= p.group_pad < 2 * kv_mul
         assert p.waves_per_group in (1, 2, 4, 8) and p.group_pad * p.waves_per_group <= 64
         if waves:

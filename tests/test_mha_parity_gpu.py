@@ -344,12 +344,14 @@ def test_workspace_laid_out_by_package_side(oracle, dev, n_q, ctx, splits, offse
 
 def test_workspace_side_falls_back_to_the_plain_layout(oracle, dev):
     """Where the layout by side does not apply -- unknown sides, a workspace without room for two homes per row, a KV
-    head count that is no multiple of eight, the separate combine kernel, a single pass -- the call runs as before."""
+    head count that is no multiple of eight, the separate combine kernel, a single pass, a wave count other than the
+    dispatcher's own -- the call runs as before."""
     case = synth.make_case(77, n_q=32, n_kv=8, ctx=4096)
     ref = run_oracle(oracle, case)
     small = 32 * 32 * 528 + 16  # exactly the plain layout's need at 32 splits
     for kw in (dict(workspace_side=0), dict(workspace_side=1, workspace_bytes=small, num_splits=32),
-               dict(workspace_side=1, force_path=B.PATH_SPLIT, num_splits=32), dict(workspace_side=1, force_path=B.PATH_SINGLE_PASS)):
+               dict(workspace_side=1, force_path=B.PATH_SPLIT, num_splits=32), dict(workspace_side=1, force_path=B.PATH_SINGLE_PASS),
+               dict(workspace_side=1, waves_per_group=2), dict(workspace_side=1, waves_per_group=8)):
         got16, _, plan = run_hip(case, dev, want_plan=True, kv_layout=B.KV_LAYOUT_HEAD_MAJOR, **kw)
         assert plan.workspace_side == 0
         assert_parity(got16, ref, str(kw))
