@@ -117,8 +117,9 @@ typedef struct llmi_mha_plan {
     int32_t waves_per_group;
     int32_t group_pad;        /* query heads per KV head rounded up to 1,2,4,8,16        */
     int32_t workspace_side;   /* 1 if the launch lays the workspace out by package side (args->workspace_side
-                                 set, fused combine, a multiple of eight KV heads, one wavefront per query head
-                                 of a group, room for two homes per row), else 0            */
+                                 set, fused combine, a multiple of eight KV heads, groups of at most 8 query
+                                 heads at the wave count the dispatcher picks itself, room for two homes per
+                                 row), else 0                                             */
     size_t workspace_needed;  /* bytes of workspace this plan uses (0 for single-pass)   */
 } llmi_mha_plan;
 
