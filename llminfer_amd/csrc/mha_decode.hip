@@ -937,14 +937,16 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             if (!all_in) __builtin_amdgcn_s_sleep(2);
         }
         if constexpr (BYSIDE) {
-            for (int spin = near_rounds; spin < a.max_polls && !all_in; ++spin) {
-                all_in = poll_round(std::true_type{});
-                if (!all_in) __builtin_amdgcn_s_sleep(2);
+            if (__builtin_expect(!all_in, 0)) {
+                for (int spin = near_rounds; spin < a.max_polls && !all_in; ++spin) {
+                    all_in = poll_round(std::true_type{});
+                    if (!all_in) __builtin_amdgcn_s_sleep(2);
+                }
             }
         }
         const bool arrived = __all(ok);
         // A give-up is counted where the host can read it (llmi_hip_poll_timeouts).
-        if (!arrived && lane == 0) atomicAdd(&g_poll_timeouts, 1u);
+        if (__builtin_expect(!arrived, 0) && lane == 0) atomicAdd(&g_poll_timeouts, 1u);
         return arrived;
     };
     // From the polled (max, sum) pairs: M = max m_s, the weights e^(m_s - M) into the head's row
@@ -988,7 +990,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     const __amdgpu_buffer_rsrc_t ws_rsrc = part_rsrc;
     constexpr int kCoherent = kCacheDevice;
 
-    if (a.group <= NW) {
+    if (G <= NW || a.group <= NW) {  // (G, the group rounded up, decides it at compile time where it can)
         // One wavefront per head, all the way: poll, then read the head's partials back and write
         // its 128 outputs, without a workgroup barrier (a wave whose records are in need not wait
         // for the others). Lane = (16-byte column, half of the splits); the two halves are added
@@ -1069,7 +1071,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 return sum;
             };
             f32x4 acc;
-            if constexpr (BYSIDE) acc = mixed ? gather(std::true_type{}) : gather(std::false_type{});
+            if constexpr (BYSIDE) acc = __builtin_expect(mixed, 0) ? gather(std::true_type{}) : gather(std::false_type{});
             else acc = gather(std::false_type{});
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = halves_sum(acc[e]);
@@ -1114,9 +1116,10 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 }
             }
         };
-        if (SA <= 16) run(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
-        else if (SA <= 64) run(std::integral_constant<int, 1>{}, std::integral_constant<int, 16>{});
-        else run(std::integral_constant<int, kMaxSplits / 64>{}, std::integral_constant<int, 16>{});
+        // (the dispatcher's own split counts stay below 64: the rare cases are kept out of the way of the usual ones)
+        if (__builtin_expect(SA > 64, 0)) run(std::integral_constant<int, kMaxSplits / 64>{}, std::integral_constant<int, 16>{});
+        else if (SA <= 16) run(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
+        else run(std::integral_constant<int, 1>{}, std::integral_constant<int, 16>{});
         return;
     }
 
