@@ -663,6 +663,34 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
 #pragma unroll
     for (int s0 = 0; s0 < NSTAGE; ++s0)
         if (s0 < n_my) issue_tile(tile_of(s0), s0);
+    // What the end of the kernel needs to know about where its results go is worked out here, while the first tiles
+    // are on their way and the wavefront has nothing else to do: behind the last tile every instruction is on the
+    // path of whoever waits for this split (the empty asm statements keep the compiler from moving the work there).
+    const bool fused = a.records != nullptr && n_active > 1;
+    const int my_xs = package_side<BYSIDE>();  // wave-uniform: the side of the package this workgroup runs on
+    // (testing aid: pretend this split ran on the other side; never the merging one, whose own rows it reads itself)
+    const int store_xs = my_xs ^ (int)(BYSIDE && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
+    const int n_units = a.group * (kHeadDim / 4);
+    const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
+    const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.ws, 0, (int)(part_rows * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
+    // A (head, 16-byte column) unit of the final merge: where its partial row and its record go.
+    struct MergeUnit {
+        int hq;
+        int64_t po;               // element offset of the column in the partial array
+        unsigned long long* rec;  // the head's record of this split (fused combine)
+    };
+    auto merge_unit = [&](int u) {
+        const int h = u >> 5, c4 = u & 31;
+        MergeUnit m;
+        m.hq = kvh * a.group + h;
+        const WsHead wh = ws_head<BYSIDE>(a, m.hq);
+        m.po = (fused ? (int64_t)ws_row<4>(wh, split, store_xs) : (int64_t)m.hq * a.num_splits + split) * kHeadDim + c4 * 4;
+        m.rec = a.records + (int64_t)ws_row<9>(wh, split, store_xs) * 2;  // (only dereferenced when fused)
+        return m;
+    };
+    MergeUnit first_unit = merge_unit((int)threadIdx.x);
+    asm volatile("" : "+v"(first_unit.hq), "+v"(first_unit.po), "+v"(first_unit.rec));
     // Query group as the MFMA B operand (zero columns beyond the group; rows beyond it
     // were filled with copies of its last row).
     {
@@ -775,19 +803,13 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     }
     __syncthreads();
 
-    const bool fused = a.records != nullptr && n_active > 1;
-    const int my_xs = package_side<BYSIDE>();  // wave-uniform: the side of the package this workgroup runs on
-    // (testing aid: pretend this split ran on the other side; never the merging one, whose own rows it reads itself)
-    const int store_xs = my_xs ^ (int)(BYSIDE && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     if constexpr (OPROJ) proj.worker = split != n_active - 1;
     // One thread per (head, 16-byte column): weights e^(m_w - M) of the waves, weighted sum.
-    const int n_units = a.group * (kHeadDim / 4);
-    const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
-    const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        a.ws, 0, (int)(part_rows * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
     for (int u = threadIdx.x; u < n_units; u += NW * 64) {
         const int h = u >> 5;
         const int c4 = u & 31;
+        MergeUnit unit = first_unit;  // (worked out while the first tiles were on their way)
+        if (u != (int)threadIdx.x) unit = merge_unit(u);
         float mw[NW];
         float mx = -INFINITY;
 #pragma unroll
@@ -803,7 +825,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             acc += *reinterpret_cast<const f32x4*>(s_o(w, h) + c4 * 4) * f;
             lsum += s_l[w][h] * f;
         }
-        const int hq = kvh * a.group + h;
+        const int hq = unit.hq;
         if (n_active == 1) {
             f32x4 r;
 #pragma unroll
@@ -816,8 +838,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
             }
         } else {
             const int64_t S = a.num_splits;
-            const WsHead wh = ws_head<BYSIDE>(a, hq);
-            const int64_t po = (fused ? (int64_t)ws_row<4>(wh, split, store_xs) : (int64_t)hq * S + split) * kHeadDim + c4 * 4;  // element offset in the workspace
+            const int64_t po = unit.po;  // element offset in the workspace
             if (fused) {
                 // Device-coherent store (cache policy sc1): it goes past this XCD's L2, so the
                 // workgroup (possibly on another XCD) that does the combine can read it without
@@ -830,7 +851,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                     // workgroup barrier is needed.
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     if (c4 == 0) {
-                        unsigned long long* rec = a.records + (int64_t)ws_row<9>(wh, split, store_xs) * 2;
+                        unsigned long long* rec = unit.rec;
                         const unsigned long long tag = a.tag;
                         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, mx);
                         const unsigned long long l_bits = __builtin_bit_cast(uint32_t, lsum);
