@@ -25,10 +25,10 @@ thread_local std::string g_last_error;
 // split over the 256 CUs. (The reference's threshold is 128 with 32-position
 // splits, mha_kernel.cu:507-517. Here the split path pays three dependent
 // memory round trips for its combine, while one workgroup streams a whole KV
-// head of 13 tiles in about 4.9 us: measured at 32 query / 8 KV heads under graph
-// replay, single pass 4.90 vs split 5.03 us at 208 positions, 5.01 vs 5.05 us at 224,
-// 5.28 vs 4.79 us at 256.)
-constexpr int kSinglePassMaxLen = 208;
+// head of 11 tiles in about 4.4 us: measured at 32 query / 8 KV heads under graph
+// replay, single pass against 8 splits 4.28 : 4.37 us at 160 positions, 4.41 : 4.45 at 176,
+// 4.53 : 4.43 at 192, 4.73 : 4.53 at 208, 5.09 : 4.36 at 256.)
+constexpr int kSinglePassMaxLen = 176;
 // Workgroups the split path aims for: one per CU (256 CUs). Each workgroup keeps
 // waves x stages x 8 KiB of loads in flight on its own; more, smaller splits only
 // add partial-result traffic and lengthen the combine (measured, ctx 1K..32K).

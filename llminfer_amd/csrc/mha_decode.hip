@@ -672,13 +672,14 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     const int store_xs = my_xs ^ (int)(BYSIDE && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     const int n_units = a.group * (kHeadDim / 4);
     const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
-    const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        a.ws, 0, (int)(part_rows * kHeadDim * (int64_t)sizeof(float)), 0x00020000);
+    int part_bytes = (int)(part_rows * kHeadDim * (int64_t)sizeof(float));
+    asm volatile("" : "+s"(part_bytes));
+    const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(a.ws, 0, part_bytes, 0x00020000);
     // A (head, 16-byte column) unit of the final merge: where its partial row and its record go.
     struct MergeUnit {
         int hq;
         int64_t po;               // element offset of the column in the partial array
-        unsigned long long* rec;  // the head's record of this split (fused combine)
+        int64_t rec;              // index of the first word of the head's record of this split (fused combine)
     };
     auto merge_unit = [&](int u) {
         const int h = u >> 5, c4 = u & 31;
@@ -686,7 +687,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         m.hq = kvh * a.group + h;
         const WsHead wh = ws_head<BYSIDE>(a, m.hq);
         m.po = (fused ? (int64_t)ws_row<4>(wh, split, store_xs) : (int64_t)m.hq * a.num_splits + split) * kHeadDim + c4 * 4;
-        m.rec = a.records + (int64_t)ws_row<9>(wh, split, store_xs) * 2;  // (only dereferenced when fused)
+        m.rec = (int64_t)ws_row<9>(wh, split, store_xs) * 2;
         return m;
     };
     MergeUnit first_unit = merge_unit((int)threadIdx.x);
@@ -810,26 +811,30 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         const int c4 = u & 31;
         MergeUnit unit = first_unit;  // (worked out while the first tiles were on their way)
         if (u != (int)threadIdx.x) unit = merge_unit(u);
-        float mw[NW];
-        float mx = -INFINITY;
+        // (all of a unit's LDS reads are requested before the first is used: one round trip, not two)
+        float mw[NW], lw[NW];
+        f32x4 ow[NW];
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             mw[w] = s_m[w][h];
-            mx = fmaxf(mx, mw[w]);
+            lw[w] = s_l[w][h];
+            ow[w] = *reinterpret_cast<const f32x4*>(s_o(w, h) + c4 * 4);
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) mx = fmaxf(mx, mw[w]);
         f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
         float lsum = 0.0f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             const float f = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - mx);
-            acc += *reinterpret_cast<const f32x4*>(s_o(w, h) + c4 * 4) * f;
-            lsum += s_l[w][h] * f;
+            acc += ow[w] * f;
+            lsum += lw[w] * f;
         }
         const int hq = unit.hq;
         if (n_active == 1) {
-            f32x4 r;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) r[e] = acc[e] / lsum;
+            const f32x4 r = acc * (1.0f / lsum);  // (one division, like the fused combine's)
             *reinterpret_cast<uint2*>(a.out + (int64_t)hq * kHeadDim + c4 * 4) = make_uint2(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]));
             if (a.out_f32) {
                 float* of = a.out_f32 + (int64_t)hq * kHeadDim + c4 * 4;  // only 4-byte alignment is promised
@@ -851,7 +856,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                     // workgroup barrier is needed.
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     if (c4 == 0) {
-                        unsigned long long* rec = unit.rec;
+                        unsigned long long* rec = a.records + unit.rec;
                         const unsigned long long tag = a.tag;
                         const unsigned long long m_bits = __builtin_bit_cast(uint32_t, mx);
                         const unsigned long long l_bits = __builtin_bit_cast(uint32_t, lsum);

@@ -107,13 +107,13 @@ def test_null_arguments():
 
 
 def test_plan_short_context_is_single_pass():
-    for pos in (0, 15, 16, 127, 159, 207):  # up to 208 positions: one workgroup per KV head
+    for pos in (0, 15, 16, 127, 159, 175):  # up to 176 positions: one workgroup per KV head
         rc, p = plan(good_args(pos=pos, workspace=0, workspace_bytes=0))  # no workspace needed
         assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1 and p.workspace_needed == 0
         assert p.rows_per_split >= pos + 1 and p.rows_per_split % 16 == 0
 
 
-@pytest.mark.parametrize("ctx", [209, 1024, 4096, 8192, 32768, 131072])
+@pytest.mark.parametrize("ctx", [177, 209, 1024, 4096, 8192, 32768, 131072])
 def test_plan_long_context_splits_without_empty_splits(ctx):
     rc, p = plan(good_args(pos=ctx - 1, max_seq_len=ctx))
     assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and 2 <= p.num_splits <= 256

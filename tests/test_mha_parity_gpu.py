@@ -80,7 +80,7 @@ def test_split_sweep_long_context_matches_oracle(oracle, dev, ctx, splits):
     assert_tap_parity(got32, ref, what)
 
 
-@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 159, 160, 161, 207, 208, 209, 239, 240, 241, 255, 256, 257, 287, 288, 289, 1000, 4097])
+@pytest.mark.parametrize("ctx", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 159, 160, 161, 175, 176, 177, 207, 208, 209, 239, 240, 241, 255, 256, 257, 287, 288, 289, 1000, 4097])
 @pytest.mark.parametrize("path", [B.PATH_SINGLE_PASS, B.PATH_SPLIT, B.PATH_SPLIT_FUSED])
 def test_ragged_lengths(oracle, dev, ctx, path):
     """Lengths around the 16-row tile, the wave count and the dispatch threshold; the cache rows past
