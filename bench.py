@@ -502,7 +502,7 @@ def run_placement(args):
     for wgs in (128, 256, 512):
         for exclusive in (0, 1):
             ids.zero_()
-            B.check(B.lib().llmi_hip_probe_placement(wgs, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream), "placement probe")
+            B.check(B.diag_lib().llmi_diag_placement(wgs, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream), "placement probe")
             torch.cuda.synchronize()
             a = ids[:2 * wgs].cpu().numpy().astype("uint32").reshape(-1, 2)
             per_cu = collections.Counter((int(x), (int(h) >> 8) & 0xFF) for x, h in a)
@@ -529,7 +529,7 @@ def run_handover_probe(args):
                 for ld in range(5):
                     reps = []
                     for _ in range(3):
-                        B.check(B.lib().llmi_hip_probe_handover(st, ld, 0, reader, precache, line.data_ptr(), res_d.data_ptr(),
+                        B.check(B.diag_lib().llmi_diag_handover(st, ld, 0, reader, precache, line.data_ptr(), res_d.data_ptr(),
                                                                torch.cuda.current_stream().cuda_stream), "handover probe")
                         torch.cuda.synchronize()
                         r = res_d.cpu().numpy()

@@ -46,7 +46,10 @@
 extern "C" {
 #endif
 
-#define LLMI_HIP_ABI_VERSION 2
+/* Bumped whenever a struct below changes size or layout, or an entry point changes meaning: a caller compiled
+ * against another value must not call into this library (llmi_hip_abi_version() returns the library's).
+ * 3: llmi_mha_args.workspace_side, llmi_mha_plan.workspace_side, llmi_attn_oproj_args.one_launch. */
+#define LLMI_HIP_ABI_VERSION 3
 
 typedef enum llmi_status {
     LLMI_OK = 0,
@@ -175,17 +178,25 @@ typedef struct llmi_attn_oproj_args {
     const void* o_weight;      /* device bf16 [hidden][head_num*128] row-major: the layer's output projection         */
     void* residual;            /* device bf16 [hidden]: residual += o_weight . attention output, rounded once          */
     int32_t hidden;
+    int32_t one_launch;        /* 0 (default): two launches, attention then projection. 1: ask for the one-launch form
+                                  (see below); only for a GPU the caller has to itself                                   */
 } llmi_attn_oproj_args;
 
 /* llmi_hip_mha_decode_append followed by llmi_hip_gemv in LLMI_GEMV_ADD_BF16 mode on its output: the tail of the
  * reference's attention block, mha_kernel_cu then fused_gemv_add_kernel_cu (code/source/model/qwen3_fused.cpp:548-552;
- * kernels mha_kernel.cu:440-529, matmul_kernel.cu:174-208) -- as ONE launch where the shape allows it. In that launch
- * the workgroups that have handed their partial results over fetch the projection's weight rows while the combine
- * still runs, wait (bounded, like the combine: llmi_hip_set_poll_limit, NaN on give-up) for the attention output and
- * finish residual += W x. Same results as the two calls, bit for bit. The one-launch form needs: the fused split path
- * with at least two splits and a host-side position, a query group of 1, 2, 4 or 8 heads, head_num*128 <= 4096,
- * hidden <= 3 * (wavefronts of the workgroups that do not combine), a grid that fits the device's compute units at
- * once, and head_num*4 more bytes of workspace than the plan reports. Anything else runs as the two launches.
+ * kernels mha_kernel.cu:440-529, matmul_kernel.cu:174-208). By default exactly those two launches (the faster form on
+ * an MI355X, and one that waits for nothing). With `one_launch` = 1, and where the shape allows it, ONE launch: the
+ * workgroups that have handed their partial results over fetch the projection's weight rows while the combine still
+ * runs, wait (bounded, like the combine: llmi_hip_set_poll_limit) for the attention output and finish
+ * residual += W x. Same results as the two calls, bit for bit. In that form workgroups wait for other workgroups of
+ * the same launch, so every workgroup of the grid has to be resident at once: ask for it only on a GPU that runs
+ * nothing else at the time (another stream's or process's kernel that holds compute units can keep the waited-for
+ * workgroups out until the wait gives up). A wait that gives up leaves its rows of the residual as they were (no
+ * NaN is stored into the in-place residual stream; the attention output is still poisoned by the combine's own
+ * give-up) and is counted: check llmi_hip_poll_timeouts. The one-launch form needs: the fused split path with at
+ * least two splits and a host-side position, a query group of 1, 2, 4 or 8 heads, head_num*128 <= 4096,
+ * hidden <= 3 * (wavefronts of the workgroups that do not combine), a grid no larger than the device's compute unit
+ * count, and head_num*4 more bytes of workspace than the plan reports. Anything else runs as the two launches.
  * llmi_hip_mha_oproj_launches tells which: 1 or 2 (or a negative status for invalid arguments). */
 int llmi_hip_mha_decode_append_oproj(const llmi_attn_oproj_args* args);
 int llmi_hip_mha_oproj_launches(const llmi_attn_oproj_args* args);
@@ -343,14 +354,6 @@ int llmi_hip_abi_version(void);
  * after the call; returns the previous limit. 0 makes every fused launch give up at once: the way to
  * exercise the failure path in a test. */
 int32_t llmi_hip_set_poll_limit(int32_t polls);
-/* No counterpart in the reference; a testing aid like the one above. With the workspace laid out by package side a
- * split keeps its partial results and record in the home near its own XCD, and the workgroup that merges finds them in
- * the home near itself because both run on one XCD. `mode` 1 makes every split but the merging one use the OTHER home,
- * mode 2 every second split: what a launch would look like whose workgroups were not dealt to the XCDs as expected.
- * The merging workgroup must then find the records by its fall-back (both homes, after 16 rounds of polls) and read
- * every split's partial results from the right home: same result, a few microseconds later. 0 (the default) switches
- * it off. Applies to launches enqueued after the call; returns the previous mode. */
-int32_t llmi_hip_set_test_far_home(int32_t mode);
 /* No counterpart in the reference. How many of those bounded waits have given up on the current device since
  * the library was loaded (one count per query head and call; the NaN outputs are the other sign). Reads a
  * device counter with a synchronous copy: it waits for work already enqueued on the device and must not be

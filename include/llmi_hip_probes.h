@@ -1,8 +1,8 @@
 /*
  * llmi_hip_probes.h -- measurement kernels of libllmi_hip.so. They have no counterpart in the reference
  * and compute nothing a model needs: bench.py uses them to put a floor under the decode-attention
- * figures (what the machine does with the same bytes when nothing is computed), to calibrate HBM byte
- * counters, and to show how a value written by one workgroup becomes visible to another.
+ * figures (what the machine does with the same bytes when nothing is computed) and to calibrate HBM byte
+ * counters; llmi_hip_mha_workspace_side decides on the ping-pong probe.
  * Same conventions as llmi_hip.h: plain pointers and sizes, LLMI_OK or a negative llmi_status, nothing
  * allocated, everything enqueued on the caller's stream.
  */
@@ -42,31 +42,6 @@ int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream);
  * every number arrived, [5] = the XCD of the pair's second workgroup. `out`: 64 uint32 of device memory. Both blocks and
  * `out` are overwritten. What llmi_hip_mha_workspace_side decides on. */
 int llmi_hip_probe_block_pingpong(void* a, void* b, uint32_t* out, void* stream);
-
-/* Where the workgroups of a launch land. `workgroups` (1..4096) workgroups of 256 threads with the LDS footprint of a
- * decode workgroup (66 KiB; `exclusive` != 0: 84 KiB, more than half a CU's LDS, so that no two share a CU) each write
- * ids[2*i] = the XCD and ids[2*i+1] = the hardware id register (HW_REG_HW_ID: CU, shader array and shader engine in
- * bits 8..15) of the CU they run on, and keep that CU for 5 us. `ids`: 2 * workgroups uint32 of device memory. */
-int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* ids, void* stream);
-
-/* Cache policy of one 4-byte load or store of the hand-over probe: the instruction's sc0 / sc1 / nt bits. */
-enum { LLMI_PROBE_PLAIN = 0, LLMI_PROBE_SC0 = 1, LLMI_PROBE_SC1 = 2, LLMI_PROBE_SC0_SC1 = 3, LLMI_PROBE_NT = 4 };
-
-typedef struct llmi_probe_handover_result {
-    uint32_t seen;      /* 1: the reader saw the writer's value within its poll budget                      */
-    uint32_t polls;     /* polls the reader made before it saw the value (or its budget, 4000)              */
-    uint32_t ns;        /* reader's time from "I am polling" to "seen", 10 ns resolution; includes the
-                           2 us the writer waits on purpose before it stores                                */
-    uint32_t xcc_reader, xcc_writer; /* XCD each side ran on (hardware id register)                        */
-} llmi_probe_handover_result;
-
-/* One writer workgroup (`writer_workgroup`, 0..15, of a grid of 16) stores a value with `store_policy`, one reader
- * workgroup (`reader_workgroup`, 0..15, another one) polls for it with `load_policy`, a bounded number of times. When
- * workgroups are dealt to the XCDs in turn, workgroups w and w + 8 share an XCD and w + 1 is on the next one. With
- * `precache` the reader has read the line before the writer writes, so stale copies exist in its L1 and L2. `line` is
- * 4 KiB of device scratch, `result` device memory; both are overwritten. Every loop in the kernel is bounded. */
-int llmi_hip_probe_handover(int32_t store_policy, int32_t load_policy, int32_t writer_workgroup, int32_t reader_workgroup,
-                            int32_t precache, void* line, llmi_probe_handover_result* result, void* stream);
 
 #ifdef __cplusplus
 }

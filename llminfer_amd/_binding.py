@@ -43,7 +43,7 @@ class MhaAppendArgs(ctypes.Structure):
 
 
 class AttnOprojArgs(ctypes.Structure):
-    _fields_ = [("attn", MhaAppendArgs), ("o_weight", c_void_p), ("residual", c_void_p), ("hidden", c_i32)]
+    _fields_ = [("attn", MhaAppendArgs), ("o_weight", c_void_p), ("residual", c_void_p), ("hidden", c_i32), ("one_launch", c_i32)]
 
 
 class GemvArgs(ctypes.Structure):
@@ -81,10 +81,10 @@ class QkNormRopeArgs(ctypes.Structure):
     ]
 
 
-PROBE_PLAIN, PROBE_SC0, PROBE_SC1, PROBE_SC0_SC1, PROBE_NT = range(5)  # llmi_hip_probes.h: cache policy of the hand-over probe
+DIAG_PLAIN, DIAG_SC0, DIAG_SC1, DIAG_SC0_SC1, DIAG_NT = range(5)  # llmi_hip_diag.h: cache policy of the hand-over probe
 
 
-class ProbeHandoverResult(ctypes.Structure):
+class DiagHandoverResult(ctypes.Structure):
     _fields_ = [(n, ctypes.c_uint32) for n in ("seen", "polls", "ns", "xcc_reader", "xcc_writer")]
 
 
@@ -126,20 +126,30 @@ SYMBOLS = {
     "llmi_hip_memset_zero": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, c_i32]),
     "llmi_hip_abi_version": (ctypes.c_int, []),
     "llmi_hip_set_poll_limit": (c_i32, [c_i32]),
-    "llmi_hip_set_test_far_home": (c_i32, [c_i32]),
     "llmi_hip_poll_timeouts": (ctypes.c_int, [ctypes.POINTER(ctypes.c_uint64)]),
     # include/llmi_hip_probes.h
     "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_stream_read_rows": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
-    "llmi_hip_probe_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
-    "llmi_hip_probe_placement": (ctypes.c_int, [c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_block_pingpong": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "llmi_hip_last_error": (ctypes.c_char_p, []),
+    # include/llmi_hip_testing.h
+    "llmi_hip_set_test_far_home": (c_i32, [c_i32]),
+    "llmi_hip_side_from_pingpong": (c_i32, [ctypes.POINTER(ctypes.c_uint32)]),
+    "llmi_hip_side_agreement": (c_i32, [ctypes.POINTER(c_i32), c_i32, ctypes.POINTER(c_i32)]),
+    "llmi_hip_workspace_side_stats": (None, [ctypes.POINTER(ctypes.c_uint64)]),
+}
+
+# include/llmi_hip_diag.h: the diagnostic probes, a library of their own (libllmi_diag.so)
+DIAG_LIB_PATH = os.path.join(HERE, "libllmi_diag.so")
+DIAG_SYMBOLS = {
+    "llmi_diag_handover": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p, c_void_p]),
+    "llmi_diag_placement": (ctypes.c_int, [c_i32, c_i32, c_void_p, c_void_p]),
 }
 
 _lib = None
+_diag = None
 
 
 class LlmiError(RuntimeError):
@@ -173,6 +183,22 @@ def lib():
             fn.argtypes = argtypes
         _lib = L
     return _lib
+
+
+def diag_lib():
+    """The loaded libllmi_diag.so (diagnostic probes; nothing on the product path needs it)."""
+    global _diag
+    if _diag is None:
+        lib()  # (torch's HIP runtime first, as above)
+        if not os.path.exists(DIAG_LIB_PATH):
+            raise RuntimeError("libllmi_diag.so is not built (%s missing); run `python -m llminfer_amd.build`." % DIAG_LIB_PATH)
+        L = ctypes.CDLL(DIAG_LIB_PATH)
+        for name, (restype, argtypes) in DIAG_SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _diag = L
+    return _diag
 
 
 def check(status, where):

@@ -9,8 +9,11 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libllmi_hip.so")
 HOST_LIB_PATH = os.path.join(HERE, "libllmi_host.so")
+DIAG_LIB_PATH = os.path.join(HERE, "libllmi_diag.so")
 
-HIP_SOURCES = ["mha_decode.hip", "qk_norm_rope.hip", "gemv.hip", "probes.hip", "c_api.cpp", "pool.cpp"]
+HIP_SOURCES = ["mha_decode_group4.hip", "mha_decode_group8.hip", "mha_decode_group16.hip", "mha_decode_group2.hip", "mha_decode_group1.hip",
+               "mha_decode.hip", "qk_norm_rope.hip", "gemv.hip", "probes.hip", "c_api.cpp", "pool.cpp"]
+DIAG_SOURCES = ["diag_probes.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops.
 HIPCC_FLAGS = [
@@ -42,22 +45,57 @@ def kernels_using_scratch(compiler_output):
     return bad
 
 
-def build_hip_library(verbose=False, defines=(), output=None):
-    """`defines`: extra NAME=VALUE macros (the kernels' build-time switches, e.g. LLMI_PV_VALU=1);
-    `output`: where to write a variant build instead of the in-tree library."""
+def _compile_objects(sources, defines, tag):
+    """Each source to an object file (in parallel: the kernels' file takes minutes, the others seconds), the
+    compiler's remarks of all of them joined."""
+    from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage"] + ["-D" + d for d in defines]
-    cmd += ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
-    cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES] + ["-o", output or LIB_PATH]
-    out = _run(cmd)
+    obj_dir = os.path.join(HERE, "build", tag)
+    os.makedirs(obj_dir, exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+
+    def one(src):
+        obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+        cmd = [hipcc] + flags + ["-c", "-Rpass-analysis=kernel-resource-usage"] + ["-D" + d for d in defines]
+        cmd += ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC, src, "-o", obj]
+        return obj, _run(cmd)
+
+    with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
+        results = list(pool.map(one, sources))
+    return [o for o, _ in results], "\n".join(out for _, out in results)
+
+
+def _link_shared(objects, output):
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", output])
+    return output
+
+
+def _check_remarks(out, verbose):
     bad = kernels_using_scratch(out)
     if bad:
         raise RuntimeError("kernels with a private (scratch) segment: %s" % ", ".join(sorted(set(bad))))
     # (the remarks themselves are not worth printing: a dozen lines for each of a hundred kernels)
-    out = "\n".join(l for l in out.splitlines() if "-Rpass-analysis" not in l and not re.match(r"^\s*\d*\s*\|", l))
+    out = "\n".join(l for l in out.splitlines() if "-Rpass-analysis" not in l and not re.match(r"^\s*\d*\s*\|", l)
+                    and not l.startswith("In file included from"))
     if verbose and out.strip():
         print(out)
-    return output or LIB_PATH
+
+
+def build_hip_library(verbose=False, defines=(), output=None):
+    """`defines`: extra NAME=VALUE macros (the kernels' build-time switches, e.g. LLMI_PV_VALU=1);
+    `output`: where to write a variant build instead of the in-tree library."""
+    tag = "hip" if not (defines or output) else "variant_" + re.sub(r"[^A-Za-z0-9_.-]", "_", os.path.basename(output or "x"))
+    objects, out = _compile_objects([os.path.join(CSRC, s) for s in HIP_SOURCES], list(defines), tag)
+    _check_remarks(out, verbose)
+    return _link_shared(objects, output or LIB_PATH)
+
+
+def build_diag_library(verbose=False):
+    """libllmi_diag.so: the two diagnostic probes (include/llmi_hip_diag.h), a library of their own."""
+    objects, out = _compile_objects([os.path.join(CSRC, "diag", s) for s in DIAG_SOURCES], [], "diag")
+    _check_remarks(out, verbose)
+    return _link_shared(objects, DIAG_LIB_PATH)
 
 
 def build_host_library(verbose=False):
@@ -77,7 +115,7 @@ def build_host_library(verbose=False):
 
 
 def build_all(verbose=False):
-    paths = [build_hip_library(verbose)]
+    paths = [build_hip_library(verbose), build_diag_library(verbose)]
     host = build_host_library(verbose)
     if host:
         paths.append(host)

@@ -8,6 +8,7 @@
 #include <atomic>
 #include <chrono>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -48,6 +49,32 @@ inline int pow2_floor(int x) {
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Tuning overrides from the environment, read once per process (the reference's counterparts are the compile-time
+// constants of its dispatcher, mha_kernel.cu:478,505-517): LLMI_HIP_SINGLE_PASS_MAX = longest context that still runs
+// as a single pass, LLMI_HIP_NUM_SPLITS = split count of the split path. Both apply only where the caller left the
+// choice to the dispatcher (force_path AUTO / num_splits 0); anything unparsable or out of range is ignored.
+struct EnvTuning {
+    int single_pass_max = -1;  // -1: not set
+    int num_splits = 0;        // 0: not set
+};
+int env_int(const char* name, long lo, long hi, int unset) {
+    const char* v = std::getenv(name);
+    if (!v || !*v) return unset;
+    char* end = nullptr;
+    const long x = std::strtol(v, &end, 10);
+    if (!end || *end != '\0' || x < lo || x > hi) return unset;
+    return (int)x;
+}
+const EnvTuning& env_tuning() {
+    static const EnvTuning t = [] {
+        EnvTuning e;
+        e.single_pass_max = env_int("LLMI_HIP_SINGLE_PASS_MAX", 0, 1 << 20, -1);
+        e.num_splits = env_int("LLMI_HIP_NUM_SPLITS", 2, kMaxSplits, 0);
+        return e;
+    }();
+    return t;
+}
 }  // namespace
 
 int record_hip_error(hipError_t err, const char* what) {
@@ -115,7 +142,8 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
     // Groups of 8 query heads run 8 waves per workgroup, which carry a single pass a little further
     // (64 query / 8 KV heads: single pass 5.14 us against 5.64 us split at 208 positions; at 256, where
     // 16 splits have a tile each, 5.51 against 5.34).
-    const int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 240 : kSinglePassMaxLen;
+    int single_pass_max = (group_pad == 8 && wave_cap >= 8) ? 240 : kSinglePassMaxLen;
+    if (env_tuning().single_pass_max >= 0) single_pass_max = env_tuning().single_pass_max;
     int path = a->force_path;
     if (path == LLMI_PATH_AUTO) {
         if (a->num_splits == 1) path = LLMI_PATH_SINGLE_PASS;
@@ -135,6 +163,14 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
         if (auto_waves > max_waves) auto_waves = max_waves;
         waves = a->waves_per_group ? a->waves_per_group : auto_waves;
         int want = a->num_splits;
+        const size_t per_split = fused ? per_split_fused : per_split_plain;
+        const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
+        if (want == 0 && a->force_path == LLMI_PATH_AUTO && env_tuning().num_splits) {
+            // the environment's split count, within what the caller's workspace holds
+            if (cap < 2) return LLMI_ERR_WORKSPACE;
+            want = env_tuning().num_splits;
+            if ((size_t)want > cap) want = (int)cap;
+        }
         if (want == 0) {
             // Auto: one workgroup per CU (kTargetGroups / kv heads splits) once half as many would need more
             // than a tile per wavefront; half as many below that, a quarter when even those would be left
@@ -162,8 +198,6 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             const int full = waves == 8 ? target * 16 : half * waves * per_wave + 1;
             want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
-            const size_t per_split = fused ? per_split_fused : per_split_plain;
-            const size_t cap = (a->workspace && a->workspace_bytes > 16) ? (a->workspace_bytes - 16) / per_split : 0;
             if (cap < 2) return LLMI_ERR_WORKSPACE;
             if ((size_t)want > cap) want = (int)cap;
         }
@@ -309,8 +343,10 @@ static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, boo
         if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
     if (!(ap.eps >= 0.0f) || args->hidden <= 0) return LLMI_ERR_INVALID_ARG;
     if (ap.mha.force_path == LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
+    if (args->one_launch != 0 && args->one_launch != 1) return LLMI_ERR_INVALID_ARG;
     if (int rc = make_plan(&ap.mha, plan, kMaxWaves, 1)) return rc;
     *fused = false;
+    if (!args->one_launch) return LLMI_OK;  // the pair of launches is the default: it is the faster form and waits for nothing
     const llmi_mha_args& m = ap.mha;
     const int n_kv = m.kv_dim / m.head_dim;
     int32_t rows_per_wave = 0, max_k = 0;
@@ -385,7 +421,8 @@ size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t 
     // ... and room for the layout by package side: the way to the first 8 KiB boundary, both arrays rounded up to whole
     // blocks per side; never less than what llmi_hip_mha_workspace_side needs for its measurement.
     const size_t plain = (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16;
-    const size_t by_side = fused_workspace(head_num, head_dim, splits, true).bytes() + 2 * kSideBlock;
+    // (the layout by side exists for the head_dim the kernels take; a row of any other width would not fit its 8 KiB blocks)
+    const size_t by_side = head_dim == 128 ? fused_workspace(head_num, head_dim, splits, true).bytes() + 2 * kSideBlock : 0;
     size_t need = (plain > by_side ? plain : by_side) + (size_t)head_num * sizeof(uint32_t);
     if (need < 6 * kSideBlock) need = 6 * kSideBlock;
     return need;

@@ -169,6 +169,7 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
                 t.o_weight = out_weight(layer);
                 t.residual = residual();
                 t.hidden = hidden_dim_;
+                t.one_launch = 1;  // (this mode exists to run the one-launch form; the stack has the GPU to itself)
                 rc = llmi_hip_mha_decode_append_oproj(&t);
             } else {
                 rc = llmi_hip_mha_decode_append(&f);

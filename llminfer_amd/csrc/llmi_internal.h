@@ -46,7 +46,7 @@ inline FusedWorkspace fused_workspace(int head_num, int head_dim, int num_splits
         w.record_bytes = (size_t)head_num * num_splits * rec;
     } else {
         const size_t rows = (size_t)head_num * num_splits;  // each with two homes
-        const size_t per_pblock = kSideBlock / row, per_rblock = kSideBlock / rec;
+        const size_t per_pblock = row <= kSideBlock ? kSideBlock / row : 1, per_rblock = kSideBlock / rec;  // (row = 512 bytes for the kernels' head_dim)
         w.partial_bytes = 2 * ((rows + per_pblock - 1) / per_pblock) * kSideBlock;
         w.record_bytes = 2 * ((rows + per_rblock - 1) / per_rblock) * kSideBlock;
     }

@@ -1,0 +1,79 @@
+// The argument block of the decode-attention kernels, shared by the launcher (mha_decode.hip) and the
+// translation units that instantiate the kernels (one per query-group size: mha_decode_group*.hip).
+#ifndef LLMI_MHA_DECODE_ARGS_H
+#define LLMI_MHA_DECODE_ARGS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace llmi {
+
+struct KernelArgs {
+    const uint16_t* q;    // [n_kv*group][128]
+    const uint16_t* k;    // layer base
+    const uint16_t* v;    // layer base
+    float* ws;            // split partials (num_splits > 1)
+    uint16_t* out;        // [n_kv*group][128]
+    float* out_f32;       // optional
+    unsigned long long* records;   // [n_q][num_splits][2] arrival records of the fused combine, or nullptr
+    uint32_t tag;                  // record tag of this call: see record_tag()
+    const int32_t* pos_dev;        // optional: position read at run time (seq_len then is its upper bound + 1)
+    int32_t row_stride;   // elements between consecutive positions of one KV head
+    int64_t head_stride;  // elements between KV heads
+    int32_t seq_len;
+    int32_t tiles_run, tiles_longer;  // tiles per split and how many splits take one more (position known on the host)
+    int32_t max_polls;             // polls of the fused combine before it gives up and writes NaN
+    bool stagger;                  // walk the tiles of a split from a split-dependent starting point (plain variant only)
+    int32_t group;        // query heads per KV head
+    int32_t n_q;          // query heads
+    int32_t num_splits;
+    float scale_log2e;       // log2(e) / sqrt(head_dim)
+    // Fused append (APPEND kernels only): q is the raw query; the new token's K
+    // row is normalised + rotated, its V row copied, both stored at position
+    // seq_len-1 of the cache and used from registers.
+    const uint16_t* k_new;   // [n_kv][128] raw
+    const uint16_t* v_new;   // [n_kv][128]
+    const uint16_t* norm_w;  // [2][128]: q_norm, k_norm
+    const float* sin_cache;  // [max_seq_len][64]
+    const float* cos_cache;
+    int64_t slot_head_stride;  // elements between KV heads inside a slot
+    float eps;
+    // Fused output projection (OPROJ kernels only): after the attention the workgroups that do not
+    // combine compute residual[r] += o_w[r] . out for their share of the rows.
+    uint32_t* ready;         // in the workspace: [0] generation word, [4 + hq] "head hq's output is written" = generation + 1
+    const uint16_t* o_w;     // [o_n][n_q * 128] bf16, row-major
+    uint16_t* o_res;         // [o_n] bf16 residual stream, updated in place
+    int32_t o_n;             // rows (the model's hidden size)
+    // Fused combine, by_side: every row of the partial and record arrays has a home in each 8 KiB block of a 16 KiB
+    // pair, and a workgroup uses the one near its XCD (see WsHead); else plain [head][split] arrays. Bit h of
+    // ppar / rpar (two words: 128 heads): which block of a pair (address bit 13) the XCDs 0-3 use for head h's
+    // partial outputs / records; XCDs 4-7 use the other one.
+    bool by_side;
+    unsigned long long ppar[2], rpar[2];
+    int32_t far_home;  // testing aid: 1 = every split but the merging one, 2 = every second one uses the other side's home
+};
+
+// Launchers of the kernels instantiated for a (padded) group of G query heads per KV head; each lives in its own
+// translation unit so that the groups compile side by side. `nw`: wavefronts per workgroup; false if the kernel is
+// not instantiated for that count.
+bool launch_decode_group1(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream);
+bool launch_decode_group2(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream);
+bool launch_decode_group4(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream);
+bool launch_decode_group8(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream);
+bool launch_decode_group16(const KernelArgs& ka, int n_kv, int nw, bool append, hipStream_t stream);
+// The one-launch form with the output projection: 4 wavefronts (8 for groups of 8); false otherwise.
+bool launch_oproj_group1(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream);
+bool launch_oproj_group2(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream);
+bool launch_oproj_group4(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream);
+bool launch_oproj_group8(const KernelArgs& ka, int n_kv, int nw, hipStream_t stream);
+// Give-ups of the fused combine's bounded waits counted by a unit's kernels on the current device (every unit has
+// its own device counter; read_poll_timeouts adds them up).
+hipError_t poll_timeouts_group1(unsigned int* n);
+hipError_t poll_timeouts_group2(unsigned int* n);
+hipError_t poll_timeouts_group4(unsigned int* n);
+hipError_t poll_timeouts_group8(unsigned int* n);
+hipError_t poll_timeouts_group16(unsigned int* n);
+
+}  // namespace llmi
+
+#endif

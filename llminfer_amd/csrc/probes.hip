@@ -1,12 +1,16 @@
 // Measurement kernels (declared in llmi_hip_probes.h): a stream-only reader with the decode kernel's
-// access pattern, a plain copy of known traffic, and a two-workgroup hand-over probe. Nothing here
-// is on the product path.
+// access pattern, a plain copy of known traffic, and the ping-pong probe that llmi_hip_mha_workspace_side
+// decides on (the only one of them a product call uses, once per workspace allocation).
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "llmi_hip_probes.h"
+#include "llmi_hip_testing.h"
 #include "llmi_internal.h"
+#include "side_decision.h"
 
 namespace llmi {
 namespace {
@@ -93,79 +97,14 @@ __device__ __forceinline__ uint32_t xcc_id() {
     return x & 15u;
 }
 
-template <int M>
-__device__ __forceinline__ uint32_t load_policy(const uint32_t* p) {
+// Device-scope (sc1) 4-byte load and store, each waited for: what the fused combine's hand-over uses.
+__device__ __forceinline__ uint32_t load_device_scope(const uint32_t* p) {
     uint32_t v;
-    if constexpr (M == LLMI_PROBE_PLAIN) asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    if constexpr (M == LLMI_PROBE_SC0) asm volatile("global_load_dword %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    if constexpr (M == LLMI_PROBE_SC1) asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    if constexpr (M == LLMI_PROBE_SC0_SC1) asm volatile("global_load_dword %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    if constexpr (M == LLMI_PROBE_NT) asm volatile("global_load_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
-template <int M>
-__device__ __forceinline__ void store_policy(uint32_t* p, uint32_t v) {
-    if constexpr (M == LLMI_PROBE_PLAIN) asm volatile("global_store_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-    if constexpr (M == LLMI_PROBE_SC0) asm volatile("global_store_dword %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-    if constexpr (M == LLMI_PROBE_SC1) asm volatile("global_store_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-    if constexpr (M == LLMI_PROBE_SC0_SC1) asm volatile("global_store_dword %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-    if constexpr (M == LLMI_PROBE_NT) asm volatile("global_store_dword %0, %1, off nt\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-}
-
-constexpr uint32_t kProbeValue = 42u;
-constexpr uint32_t kProbePolls = 4000u;
-
-// line[0]: the data word; line[64] (another 256-byte line): reader -> writer "I am polling".
-template <int WM, int RM>
-__global__ __launch_bounds__(64) void handover_kernel(uint32_t* line, llmi_probe_handover_result* res, int writer_wg, int reader_wg, int precache) {
-    if (threadIdx.x != 0) return;
-    uint32_t* data = line;
-    uint32_t* flag = line + 64;
-    if ((int)blockIdx.x == reader_wg) {
-        if (precache) (void)(load_policy<LLMI_PROBE_PLAIN>(data) + load_policy<RM>(data));
-        store_policy<LLMI_PROBE_SC1>(flag, 1u);
-        const unsigned long long t0 = wall_clock64();
-        uint32_t polls = 0, seen = 0;
-        for (; polls < kProbePolls; ++polls)
-            if (load_policy<RM>(data) == kProbeValue) {
-                seen = 1;
-                break;
-            }
-        const unsigned long long t1 = wall_clock64();
-        res->seen = seen;
-        res->polls = polls;
-        res->ns = (uint32_t)((t1 - t0) * 10ull);
-        res->xcc_reader = xcc_id();
-    } else if ((int)blockIdx.x == writer_wg) {
-        res->xcc_writer = xcc_id();
-        for (int i = 0; i < 200000; ++i)  // bounded: the reader raises the flag at once
-            if (load_policy<LLMI_PROBE_SC1>(flag) == 1u) break;
-        const unsigned long long t0 = wall_clock64();
-        while (wall_clock64() - t0 < 200ull) {  // 2 us: the reader is polling by now
-        }
-        store_policy<WM>(data, kProbeValue);
-    }
-}
-
-// Where the workgroups of a launch land: every workgroup (256 threads, LDS bytes of LDS: the footprint of a
-// decode workgroup, or more than half a CU's LDS so that two cannot share a CU) records the XCD and the
-// hardware id register of the CU it runs on, then keeps its CU for hold_ticks of the 100 MHz clock (bounded),
-// so that the whole grid is resident at once like the decode kernel's.
-template <int LDS>
-__global__ __launch_bounds__(256) void placement_kernel(uint32_t* out, uint32_t hold_ticks) {
-    __shared__ char pad[LDS];
-    if (threadIdx.x == 0) {
-        *reinterpret_cast<volatile char*>(pad) = 1;  // (keeps the allocation)
-        uint32_t hw;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-        out[2 * blockIdx.x] = xcc_id();
-        out[2 * blockIdx.x + 1] = hw;
-    }
-    const unsigned long long t0 = wall_clock64();
-    for (int i = 0; i < 100000; ++i) {  // bounded: 100 us at the most with the sleep below
-        if (wall_clock64() - t0 >= hold_ticks) break;
-        __builtin_amdgcn_s_sleep(8);
-    }
+__device__ __forceinline__ void store_device_scope(uint32_t* p, uint32_t v) {
+    asm volatile("global_store_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
 }
 
 // Hand-over latency from every XCD through two blocks of memory. Workgroups i and i + 8 of a grid of 16 (one XCD when
@@ -174,7 +113,7 @@ __global__ __launch_bounds__(256) void placement_kernel(uint32_t* out, uint32_t 
 // word, i polls for that. kPingPongs round trips per chain; every poll loop is bounded, a pair that loses a number
 // gives up and says so. Workgroup i < 8 reports: its XCD, its partner's, the ticks (10 ns) spent on a and on b, 1 if
 // every number arrived.
-constexpr int kPingPongs = 16, kPingPongChains = 2, kPingPongPolls = 4000;
+constexpr int kPingPongPolls = 4000;  // (kPingPongs round trips per chain, kPingPongChains chains: side_decision.h)
 __global__ __launch_bounds__(64) void block_pingpong_kernel(uint32_t* a, uint32_t* b, uint32_t* out) {
     if (threadIdx.x != 0) return;
     const int pair = blockIdx.x & 7;
@@ -193,11 +132,11 @@ __global__ __launch_bounds__(64) void block_pingpong_kernel(uint32_t* a, uint32_
                 ++seq;
                 uint32_t* mine = leader ? ping : pong;
                 const uint32_t* theirs = leader ? pong : ping;
-                if (leader) store_policy<LLMI_PROBE_SC1>(mine, seq);
+                if (leader) store_device_scope(mine, seq);
                 int polls = 0;
-                while (polls < kPingPongPolls && load_policy<LLMI_PROBE_SC1>(theirs) != seq) ++polls;
+                while (polls < kPingPongPolls && load_device_scope(theirs) != seq) ++polls;
                 if (polls == kPingPongPolls) ok = 0;
-                if (!leader) store_policy<LLMI_PROBE_SC1>(mine, seq);
+                if (!leader) store_device_scope(mine, seq);
             }
             t[which] += wall_clock64() - t0;
         }
@@ -206,18 +145,6 @@ __global__ __launch_bounds__(64) void block_pingpong_kernel(uint32_t* a, uint32_
         out[8 * pair + 1] = (uint32_t)t[0];
         out[8 * pair + 2] = (uint32_t)t[1];
         out[8 * pair + 3] = ok;
-    }
-}
-
-typedef void (*HandoverKernel)(uint32_t*, llmi_probe_handover_result*, int, int, int);
-template <int WM>
-HandoverKernel pick_reader(int rm) {
-    switch (rm) {
-        case LLMI_PROBE_PLAIN: return handover_kernel<WM, LLMI_PROBE_PLAIN>;
-        case LLMI_PROBE_SC0: return handover_kernel<WM, LLMI_PROBE_SC0>;
-        case LLMI_PROBE_SC1: return handover_kernel<WM, LLMI_PROBE_SC1>;
-        case LLMI_PROBE_SC0_SC1: return handover_kernel<WM, LLMI_PROBE_SC0_SC1>;
-        default: return handover_kernel<WM, LLMI_PROBE_NT>;
     }
 }
 
@@ -249,34 +176,28 @@ namespace llmi {
 
 // Which 8 KiB blocks lie near which side of the package, seen from the workspace itself: the time of hand-overs between
 // two workgroups of one XCD (block_pingpong_kernel, all eight XCDs at once, each pair reporting the XCD it ran on)
-// through a block with address bit 13 clear and through its neighbour with the bit set. The two sides of the package
-// must disagree about which block is nearer, each clearly: anything else is reported as "no statement" (0).
+// through a block with address bit 13 clear and through its neighbour with the bit set. One run gives one decision
+// (side_from_pingpong: the two sides of the package must disagree about which block is nearer, each clearly); the
+// answer is a side only when two runs name it and none names the other (side_agreement), else "no statement" (0).
+// What it answered is counted (llmi_hip_workspace_side_stats).
+static std::atomic<unsigned long long> g_side_stats[3];
 static int measure_window_side(char* window, hipStream_t stream, int* side) {
     *side = 0;
     // The pairs' lines: the first 2 KiB of either block; the results: the second 4 KiB of the first block.
     uint32_t* out = reinterpret_cast<uint32_t*>(window + 4096);
-    for (int attempt = 0; attempt < 3; ++attempt) {
+    constexpr int kRuns = 4;
+    int decisions[kRuns];
+    int runs = 0, verdict = kSideAbstained;
+    while (runs < kRuns) {
         if (int rc = llmi_hip_probe_block_pingpong(window, window + kSideBlock, out, stream)) return rc;
-        uint32_t r[8][8];
+        uint32_t r[64];
         if (int rc = record_hip_error(hipMemcpyAsync(r, out, sizeof(r), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync")) return rc;
         if (int rc = record_hip_error(hipStreamSynchronize(stream), "hipStreamSynchronize")) return rc;
-        long long diff[2] = {0, 0};  // per side of the package: ticks through the clear block minus ticks through the set block
-        int n[2] = {0, 0};
-        for (int p = 0; p < 8; ++p) {
-            if (!r[p][3] || r[p][0] != r[p][5]) continue;  // a pair that lost a number, or did not share an XCD
-            const int sd = (int)(r[p][0] >> 2) & 1;
-            diff[sd] += (long long)r[p][1] - (long long)r[p][2];
-            ++n[sd];
-        }
-        if (n[0] < 2 || n[1] < 2) continue;
-        // Per hand-over (two per round trip), in ns (a tick is 10 ns).
-        const long long handovers = 2ll * kPingPongs * kPingPongChains;
-        const long long d0 = diff[0] * 10 / (n[0] * handovers), d4 = diff[1] * 10 / (n[1] * handovers);
-        constexpr long long kThresholdNs = 25;
-        if (d0 <= -kThresholdNs && d4 >= kThresholdNs) *side = 1;       // XCDs 0-3 are nearer to the clear block, 4-7 to the set one
-        else if (d0 >= kThresholdNs && d4 <= -kThresholdNs) *side = 2;
-        if (*side) break;
+        decisions[runs++] = side_from_pingpong(r);
+        *side = side_agreement(decisions, runs, &verdict);
+        if (verdict != kSideAbstained) break;  // two runs agree, or two contradict each other: more runs change neither
     }
+    g_side_stats[verdict].fetch_add(1, std::memory_order_relaxed);
     return LLMI_OK;
 }
 
@@ -379,37 +300,22 @@ int llmi_hip_probe_block_pingpong(void* a, void* b, uint32_t* out, void* stream)
     return check_launch();
 }
 
-int llmi_hip_probe_placement(int32_t workgroups, int32_t exclusive, uint32_t* ids, void* stream) {
-    if (!ids) return LLMI_ERR_NULL_POINTER;
-    if (workgroups < 1 || workgroups > 4096) return LLMI_ERR_INVALID_ARG;
-    if ((uintptr_t)ids & 3u) return LLMI_ERR_ALIGNMENT;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const uint32_t hold = 500;  // 5 us
-    if (exclusive) hipLaunchKernelGGL((placement_kernel<84 * 1024>), dim3(workgroups), dim3(256), 0, s, ids, hold);
-    else hipLaunchKernelGGL((placement_kernel<66 * 1024>), dim3(workgroups), dim3(256), 0, s, ids, hold);
-    return check_launch();
+int32_t llmi_hip_side_from_pingpong(const uint32_t* results64) { return results64 ? side_from_pingpong(results64) : 0; }
+
+int32_t llmi_hip_side_agreement(const int32_t* decisions, int32_t count, int32_t* verdict) {
+    if (!decisions || count < 0) {
+        if (verdict) *verdict = kSideAbstained;
+        return 0;
+    }
+    int v = kSideAbstained;
+    const int side = side_agreement(decisions, count, &v);
+    if (verdict) *verdict = v;
+    return side;
 }
 
-int llmi_hip_probe_handover(int32_t store_pol, int32_t load_pol, int32_t writer_workgroup, int32_t reader_workgroup, int32_t precache, void* line,
-                            llmi_probe_handover_result* result, void* stream) {
-    if (!line || !result) return LLMI_ERR_NULL_POINTER;
-    if (store_pol < 0 || store_pol > LLMI_PROBE_NT || load_pol < 0 || load_pol > LLMI_PROBE_NT) return LLMI_ERR_INVALID_ARG;
-    if (writer_workgroup < 0 || writer_workgroup > 15 || reader_workgroup < 0 || reader_workgroup > 15 || writer_workgroup == reader_workgroup)
-        return LLMI_ERR_INVALID_ARG;
-    if ((uintptr_t)line & 255u) return LLMI_ERR_ALIGNMENT;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (int rc = record_hip_error(hipMemsetAsync(line, 0, 4096, s), "hipMemsetAsync")) return rc;
-    if (int rc = record_hip_error(hipMemsetAsync(result, 0, sizeof(*result), s), "hipMemsetAsync")) return rc;
-    HandoverKernel k;
-    switch (store_pol) {
-        case LLMI_PROBE_PLAIN: k = pick_reader<LLMI_PROBE_PLAIN>(load_pol); break;
-        case LLMI_PROBE_SC0: k = pick_reader<LLMI_PROBE_SC0>(load_pol); break;
-        case LLMI_PROBE_SC1: k = pick_reader<LLMI_PROBE_SC1>(load_pol); break;
-        case LLMI_PROBE_SC0_SC1: k = pick_reader<LLMI_PROBE_SC0_SC1>(load_pol); break;
-        default: k = pick_reader<LLMI_PROBE_NT>(load_pol); break;
-    }
-    hipLaunchKernelGGL(k, dim3(16), dim3(64), 0, s, static_cast<uint32_t*>(line), result, (int)writer_workgroup, (int)reader_workgroup, (int)precache);
-    return check_launch();
+void llmi_hip_workspace_side_stats(uint64_t out[3]) {
+    if (!out) return;
+    for (int i = 0; i < 3; ++i) out[i] = g_side_stats[i].load(std::memory_order_relaxed);
 }
 
 }  // extern "C"

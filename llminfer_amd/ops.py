@@ -118,9 +118,10 @@ def qk_norm_rope_append(query, key_new, value_new, key_cache, value_cache, norm_
 
 
 def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos_cache, key_cache, value_cache,
-                      output, workspace, *, eps=1e-6, stream=None, o_weight=None, residual=None, **kw):
+                      output, workspace, *, eps=1e-6, stream=None, o_weight=None, residual=None, one_launch=False, **kw):
     """QK-Norm + RoPE + K/V append + decode attention as one kernel (llmi_hip_mha_decode_append). With `o_weight`
-    [hidden][head_num*128] and `residual` [hidden]: llmi_hip_mha_decode_append_oproj; returns the launch count."""
+    [hidden][head_num*128] and `residual` [hidden]: llmi_hip_mha_decode_append_oproj (`one_launch`: ask for its
+    one-launch form); returns the launch count."""
     for name, t in (("query_raw", query_raw), ("key_new", key_new), ("value_new", value_new),
                     ("norm_weight", norm_weight), ("key_cache", key_cache), ("value_cache", value_cache),
                     ("output", output)):
@@ -140,6 +141,7 @@ def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos
     _check_dev("residual", residual, _BF16_DTYPES)
     t = B.AttnOprojArgs()
     t.attn, t.o_weight, t.residual, t.hidden = a, _ptr(o_weight), _ptr(residual), residual.numel()
+    t.one_launch = 1 if one_launch else 0
     launches = B.lib().llmi_hip_mha_oproj_launches(ctypes.byref(t))
     B.check(B.lib().llmi_hip_mha_decode_append_oproj(ctypes.byref(t)), "llmi_hip_mha_decode_append_oproj")
     return launches

@@ -502,9 +502,15 @@ def test_fused_output_projection_equals_attention_then_gemv_add(oracle, dev, n_q
     ops.gemv(out_a, wo_d.view(hidden, dim), res_a, mode=B.GEMV_ADD_BF16)
     torch.cuda.synchronize()
     assert_parity(from_dev_bf16(out_a), ref, "attention in front of the projection")
+    # the entry point's default is the same pair of launches
+    kc, vc, out_d, res_d = fresh()
+    assert ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_d, ws, o_weight=wo_d, residual=res_d, **kw) == 2
+    torch.cuda.synchronize()
+    assert torch.equal(out_d, out_a) and torch.equal(res_d, res_a)
     for call in range(3):
         kc, vc, out_b, res_b = fresh()
-        launches = ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_b, ws, o_weight=wo_d, residual=res_b, **kw)
+        launches = ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out_b, ws, o_weight=wo_d, residual=res_b,
+                                         one_launch=True, **kw)
         torch.cuda.synchronize()
         assert launches == want_launches
         # The one-launch form may ask for more splits than the dispatcher would pick on its own (it needs idle
@@ -520,6 +526,54 @@ def test_fused_output_projection_equals_attention_then_gemv_add(oracle, dev, n_q
             assert torch.equal(res_b, res_a), "call %d: residuals differ" % call
     n = ctypes.c_uint64()
     assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(n)) == 0
+
+
+def test_one_launch_projection_that_gives_up_leaves_the_residual_alone(dev):
+    """The one-launch form with the poll limit forced to zero: every wait gives up at once, every kernel still ends
+    normally, the attention output is poisoned (NaN), the in-place residual stream keeps its bits, and the give-ups are
+    counted. With the limit restored the next call on the same workspace matches the pair of launches."""
+    n_q, n_kv, d, ctx, hidden = 32, 8, 128, 4096, 2560
+    rng = np.random.RandomState(5)
+    msl, pos, kv_dim, dim = ctx + 2, ctx, n_kv * d, n_q * d
+    case = synth.make_case(901, n_q=n_q, n_kv=n_kv, ctx=ctx, max_seq_len=msl)
+    bits = lambda *shape, scale=1.0: synth.f32_to_bf16_bits((scale * rng.standard_normal(shape)).astype(np.float32))
+    q_raw, k_new, v_new = bits(n_q * d), bits(kv_dim), bits(kv_dim)
+    w = synth.f32_to_bf16_bits((1 + 0.02 * rng.standard_normal(2 * d)).astype(np.float32))
+    wo, res0 = bits(hidden * dim, scale=1 / np.sqrt(dim)), bits(hidden)
+    sin_d, cos_d = ops.sincos_table(d, msl, dev)
+    wo_d, w_d, qd, kd, vd = (to_dev(x, dev) for x in (wo, w, q_raw, k_new, v_new))
+    ws = torch.full((ops.workspace_bytes(n_q, d, msl) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    kw = dict(layer_id=0, pos=pos, kv_dim=kv_dim, kv_mul=n_q // n_kv, head_num=n_q, head_dim=d, max_seq_len=msl,
+              kv_layout=B.KV_LAYOUT_HEAD_MAJOR)
+
+    def run(one_launch):
+        kc, vc = to_dev(synth.to_head_major(case["k"], n_kv), dev), to_dev(synth.to_head_major(case["v"], n_kv), dev)
+        out, res = torch.zeros(dim, dtype=torch.int16, device=dev), to_dev(res0, dev)
+        n = ops.mha_decode_append(qd, kd, vd, w_d, sin_d, cos_d, kc, vc, out, ws, o_weight=wo_d, residual=res, one_launch=one_launch, **kw)
+        torch.cuda.synchronize()
+        return n, out, res
+
+    def timeouts():
+        n = ctypes.c_uint64()
+        assert B.lib().llmi_hip_poll_timeouts(ctypes.byref(n)) == 0
+        return n.value
+
+    _, out_pair, res_pair = run(False)
+    before = timeouts()
+    prev = B.lib().llmi_hip_set_poll_limit(0)
+    try:
+        n, out, res = run(True)
+    finally:
+        assert B.lib().llmi_hip_set_poll_limit(prev) == 0
+    assert n == 1
+    assert np.all(np.isnan(from_dev_bf16(out)))
+    assert torch.equal(res, to_dev(res0, dev)), "a give-up must not touch the residual stream"
+    assert timeouts() > before
+    after = timeouts()
+    ws.fill_(float("nan"))  # (records of the abandoned launch may have arrived late)
+    n, out, res = run(True)
+    assert n == 1 and torch.equal(res, res_pair) and timeouts() == after
+    assert_parity(from_dev_bf16(out), from_dev_bf16(out_pair), "one launch after a give-up")
 
 
 def test_mha_op_forward_through_registry_hook(oracle, dev):

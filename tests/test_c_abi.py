@@ -12,11 +12,12 @@ import pytest
 from llminfer_amd import _binding as B
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("llmi_hip.h", "llmi_hip_probes.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("llmi_hip.h", "llmi_hip_probes.h", "llmi_hip_testing.h")]
+DIAG_HEADER = os.path.join(ROOT, "include", "llmi_hip_diag.h")
 
 
-def declared_functions():
-    text = "".join(open(h).read() for h in HEADERS)
+def declared_functions(headers=HEADERS):
+    text = "".join(open(h).read() for h in headers)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b(llmi_[a-z0-9_]+)\s*\(", text)
     # typedef'd function-pointer types are not exported symbols
@@ -31,7 +32,22 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(lib, name), "libllmi_hip.so does not export " + name
         assert name in B.SYMBOLS, "the ctypes binding does not declare " + name
     assert set(B.SYMBOLS) == set(names)
-    assert lib.llmi_hip_abi_version() == 2
+    header = open(HEADERS[0]).read()
+    declared = int(re.search(r"#define\s+LLMI_HIP_ABI_VERSION\s+(\d+)", header).group(1))
+    assert declared == 3 and lib.llmi_hip_abi_version() == declared
+    # every header of include/ is covered by this test or the next one
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == sorted(os.path.basename(h) for h in HEADERS + [DIAG_HEADER])
+
+
+def test_diag_library_exports_its_header():
+    lib = B.diag_lib()
+    names = declared_functions([DIAG_HEADER])
+    assert names == sorted(B.DIAG_SYMBOLS)
+    for name in names:
+        assert hasattr(lib, name), "libllmi_diag.so does not export " + name
+    # ... and the product library carries none of it
+    for name in names + ["llmi_hip_probe_handover", "llmi_hip_probe_placement"]:
+        assert not hasattr(B.lib(), name)
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -43,6 +59,8 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
 int main(void) {
     printf("%zu %zu %zu %zu %zu\n", sizeof(llmi_mha_args), offsetof(llmi_mha_args, layer_id),
            offsetof(llmi_mha_args, waves_per_group), offsetof(llmi_mha_args, stream), sizeof(llmi_mha_plan));
+    printf("%zu %zu %zu %zu %zu\n", offsetof(llmi_mha_args, workspace_side), sizeof(llmi_mha_append_args),
+           offsetof(llmi_mha_append_args, eps), sizeof(llmi_attn_oproj_args), offsetof(llmi_attn_oproj_args, one_launch));
     printf("%zu %zu %zu %zu\n", sizeof(llmi_qk_norm_rope_args), offsetof(llmi_qk_norm_rope_args, eps),
            offsetof(llmi_qk_norm_rope_args, stream), sizeof(llmi_pool_stats));
     return 0;
@@ -53,7 +71,9 @@ int main(void) {
     out = subprocess.run([str(exe)], check=True, stdout=subprocess.PIPE, text=True).stdout.split()
     got = [int(x) for x in out]
     want = [ctypes.sizeof(B.MhaArgs), B.MhaArgs.layer_id.offset, B.MhaArgs.waves_per_group.offset,
-            B.MhaArgs.stream.offset, ctypes.sizeof(B.MhaPlan), ctypes.sizeof(B.QkNormRopeArgs),
+            B.MhaArgs.stream.offset, ctypes.sizeof(B.MhaPlan),
+            B.MhaArgs.workspace_side.offset, ctypes.sizeof(B.MhaAppendArgs), B.MhaAppendArgs.eps.offset,
+            ctypes.sizeof(B.AttnOprojArgs), B.AttnOprojArgs.one_launch.offset, ctypes.sizeof(B.QkNormRopeArgs),
             B.QkNormRopeArgs.eps.offset, B.QkNormRopeArgs.stream.offset, ctypes.sizeof(B.PoolStats)]
     assert got == want
 
@@ -320,3 +340,83 @@ def test_build_rejects_kernels_with_a_private_segment():
         "a.hip:9:1: remark:     ScratchSize [bytes/lane]: 48 [-Rpass-analysis=kernel-resource-usage]"])
     assert build.kernels_using_scratch(remarks) == ["kern_b"]
     assert build.kernels_using_scratch("") == []
+
+
+@pytest.mark.parametrize("head_dim", [64, 128, 256, 4096, 2**31 - 1])
+def test_workspace_bytes_for_any_head_dim(head_dim):
+    """The size query never divides by a block count of zero (a row wider than the 8 KiB blocks of the layout by side
+    has none): any head_dim gives a size that holds the plain layout."""
+    n = B.lib().llmi_hip_mha_workspace_bytes(32, head_dim, 4096)
+    assert n >= 32 * 256 * (head_dim * 4 + 16) + 16
+    if head_dim == 128:
+        assert n >= 2 * (32 * 256 // 16) * 8192  # two homes per row
+
+
+def test_environment_overrides_of_the_dispatch():
+    """LLMI_HIP_SINGLE_PASS_MAX and LLMI_HIP_NUM_SPLITS move the threshold and the split count where the caller
+    left both to the dispatcher, and nothing else (read once per process: a child process per setting)."""
+    code = (
+        "import ctypes, sys; sys.path.insert(0, %r)\n"
+        "from tests.test_c_abi import good_args, plan\n"
+        "out = []\n"
+        "for pos, over in ((99, {}), (299, {}), (4095, {}), (4095, dict(num_splits=8)), (299, dict(force_path=1)), (4095, dict(workspace_bytes=5 * 32 * 528 + 16))):\n"
+        "    rc, p = plan(good_args(pos=pos, **over)); out.append('%%d:%%d:%%d' %% (rc, p.path, p.num_splits))\n"
+        "print(' '.join(out))\n" % ROOT)
+
+    def run(**env):
+        e = dict(os.environ, **env)
+        return subprocess.run([sys.executable, "-c", code], check=True, stdout=subprocess.PIPE, text=True, env=e, cwd=ROOT).stdout.split()
+
+    assert run() == ["0:1:1", "0:3:16", "0:3:32", "0:3:8", "0:1:1", "0:3:5"]
+    assert run(LLMI_HIP_SINGLE_PASS_MAX="400") == ["0:1:1", "0:1:1", "0:3:32", "0:3:8", "0:1:1", "0:3:5"]
+    assert run(LLMI_HIP_SINGLE_PASS_MAX="50") == ["0:3:7", "0:3:16", "0:3:32", "0:3:8", "0:1:1", "0:3:5"]
+    assert run(LLMI_HIP_NUM_SPLITS="12") == ["0:1:1", "0:3:12", "0:3:12", "0:3:8", "0:1:1", "0:3:5"]
+    assert run(LLMI_HIP_NUM_SPLITS="junk", LLMI_HIP_SINGLE_PASS_MAX="-3") == run()
+
+
+def test_side_decision_from_injected_timings():
+    """The decision behind llmi_hip_mha_workspace_side as a pure function of the ping-pong probe's result words:
+    clear cases, noise below the threshold, ties, pairs that lost a number or did not share an XCD, a side of the
+    package without two usable pairs."""
+    lib = B.lib()
+
+    def rows(spec):
+        """spec: per pair (xcd, ticks through the clear block, ticks through the set block[, ok[, partner xcd]])"""
+        r = (ctypes.c_uint32 * 64)()
+        for p, t in enumerate(spec):
+            xcd, a, b = t[:3]
+            ok = t[3] if len(t) > 3 else 1
+            partner = t[4] if len(t) > 4 else xcd
+            r[8 * p + 0], r[8 * p + 1], r[8 * p + 2], r[8 * p + 3], r[8 * p + 5] = xcd, a, b, ok, partner
+        return r
+
+    def decide(spec):
+        return lib.llmi_hip_side_from_pingpong(rows(spec))
+
+    # 64 hand-overs per block and run, ticks of 10 ns: 25 ns per hand-over = 160 ticks
+    near, far = 3600, 4400
+    assert decide([(x, near, far) for x in range(4)] + [(x, far, near) for x in range(4, 8)]) == 1
+    assert decide([(x, far, near) for x in range(4)] + [(x, near, far) for x in range(4, 8)]) == 2
+    assert decide([(x, near, near + 100) for x in range(4)] + [(x, near + 100, near) for x in range(4, 8)]) == 0   # below the threshold
+    assert decide([(x, near, near + 160) for x in range(4)] + [(x, near + 160, near) for x in range(4, 8)]) == 1   # exactly at it
+    assert decide([(x, near, near) for x in range(8)]) == 0                                                       # a tie
+    assert decide([(x, near, far) for x in range(8)]) == 0                       # both sides prefer the same block
+    assert decide([(x, near, far) for x in range(4)] + [(x, near, near + 10) for x in range(4, 8)]) == 0          # one side unclear
+    # noise on single pairs does not flip a clear average
+    assert decide([(0, far, near), (1, near, far + 900), (2, near, far), (3, near, far)] + [(x, far, near) for x in range(4, 8)]) == 1
+    # pairs that lost a number or did not share an XCD do not count; two good pairs per side are enough
+    assert decide([(0, near, far), (1, near, far), (2, 0, 0, 0), (3, far, near, 1, 5)] + [(4, far, near), (5, far, near), (6, 9, 9, 0), (7, 1, 9999, 1, 0)]) == 1
+    assert decide([(0, near, far), (1, 0, 0, 0), (2, 0, 0, 0), (3, 0, 0, 0)] + [(x, far, near) for x in range(4, 8)]) == 0  # one pair on a side
+    assert decide([(x, near, far) for x in range(4)] + [(x, 0, 0, 0) for x in range(4, 8)]) == 0                  # one side missing
+    assert decide([(12, near, far)] * 8) == 0                                                                     # no such XCD
+    assert lib.llmi_hip_side_from_pingpong(None) == 0
+
+    def agree(ds):
+        v = ctypes.c_int32(-1)
+        arr = (ctypes.c_int32 * max(1, len(ds)))(*ds)
+        return lib.llmi_hip_side_agreement(arr, len(ds), ctypes.byref(v)), v.value
+
+    assert agree([1, 1]) == (1, 0) and agree([2, 0, 2]) == (2, 0) and agree([0, 1, 0, 1]) == (1, 0)
+    assert agree([1]) == (0, 1) and agree([0, 0, 0, 0]) == (0, 1) and agree([0, 2, 0, 0]) == (0, 1) and agree([]) == (0, 1)
+    assert agree([1, 2]) == (0, 2) and agree([1, 1, 2]) == (0, 2) and agree([0, 2, 1, 2]) == (0, 2)
+    assert agree([7, 1, -1, 1]) == (1, 0)                                                                         # junk is no statement

@@ -333,12 +333,11 @@ def test_workspace_laid_out_by_package_side(oracle, dev, n_q, ctx, splits, offse
     plain16, plain32 = run_hip(case, dev, **kw)
     assert_parity(plain16, ref, "plain layout")
     ws = torch.empty(ops.workspace_bytes(n_q, 128, ctx + 1) // 4 + offset // 4, dtype=torch.float32, device=dev)[offset // 4:]
-    measured = ops.workspace_side(ws)
-    assert measured == ops.workspace_side(ws)           # the measurement repeats
-    assert any((measured >> (2 * i)) & 3 in (1, 2) for i in range(16))
-    for side in (measured, _flip_sides(measured), 0x66666666, 0x11111111 | (2 << 2)):
+    measured = ops.workspace_side(ws)  # (0 if the timing probe made no statement on this box: then only the claims run)
+    sides = ([measured, _flip_sides(measured)] if measured else []) + [0x66666666, 0x11111111 | (2 << 2), 0x55555555, -1431655766]
+    for side in sides:
         got16, got32, plan = run_hip(case, dev, want_plan=True, workspace_side=side, **kw)
-        assert plan.workspace_side in (1, 2), "side word %x" % (side & 0xFFFFFFFF)
+        assert plan.workspace_side == 1, "side word %x" % (side & 0xFFFFFFFF)
         assert np.array_equal(got16, plain16) and np.array_equal(got32, plain32), "side word %x" % (side & 0xFFFFFFFF)
 
 
@@ -359,6 +358,25 @@ def test_workspace_side_falls_back_to_the_plain_layout(oracle, dev):
     got16, _, plan = run_hip(case, dev, want_plan=True, workspace_side=1)
     assert plan.workspace_side == 0
     assert_parity(got16, run_oracle(oracle, case), "4 KV heads")
+
+
+def test_workspace_side_measurements_never_contradict(dev):
+    """Twenty measurements of one workspace: every one that makes a statement about a region makes the same one, and the
+    library's own tally has no contradiction (two probe runs naming opposite sides). How often the probe abstains is
+    reported by the tally, not asserted: an abstention keeps the plain layout and costs nothing but time."""
+    ws = torch.empty(ops.workspace_bytes(32, 128, 32768) // 4, dtype=torch.float32, device=dev)
+    stats0 = (ctypes.c_uint64 * 3)()
+    B.lib().llmi_hip_workspace_side_stats(stats0)
+    words = [ops.workspace_side(ws) & 0xFFFFFFFF for _ in range(20)]
+    stats = (ctypes.c_uint64 * 3)()
+    B.lib().llmi_hip_workspace_side_stats(stats)
+    for region in range(16):
+        named = {(w >> (2 * region)) & 3 for w in words} - {0}
+        assert len(named) <= 1, "region %d: %s" % (region, sorted(named))
+    assert stats[2] == stats0[2], "contradicting probe runs"
+    assert stats[0] + stats[1] > stats0[0] + stats0[1]
+    print("workspace side: %d agreed, %d abstained of %d region measurements"
+          % (stats[0] - stats0[0], stats[1] - stats0[1], stats[0] + stats[1] - stats0[0] - stats0[1]))
 
 
 def test_workspace_side_argument_checks(dev):

@@ -1,6 +1,7 @@
-"""The measurement kernels of the library (include/llmi_hip_probes.h): argument checks without a GPU, and
-on a GPU that every launch shape bench.py uses runs, that the copy kernel copies and that the hand-over
-probe reports what its policies are known to do."""
+"""The measurement kernels of the library (include/llmi_hip_probes.h) and the diagnostic probes of libllmi_diag.so
+(include/llmi_hip_diag.h): argument checks without a GPU, and on a GPU that every launch shape bench.py uses runs,
+that the copy kernel copies and that the probes report what they are documented to report. Timings are printed,
+never asserted: they depend on the box."""
 import ctypes
 
 import numpy as np
@@ -36,18 +37,19 @@ def test_copy_and_handover_reject_bad_arguments():
     assert lib.llmi_hip_probe_copy(None, P, 16, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_copy(P, P, 24, None) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_copy(P, P + 4, 16, None) == B.STATUS["ALIGNMENT"]
-    assert lib.llmi_hip_probe_handover(0, 2, 0, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_block_pingpong(None, P, P, None) == B.STATUS["NULL_POINTER"]
     assert lib.llmi_hip_probe_block_pingpong(P, P + 128, P, None) == B.STATUS["ALIGNMENT"]
-    assert lib.llmi_hip_probe_placement(256, 0, None, None) == B.STATUS["NULL_POINTER"]
-    assert lib.llmi_hip_probe_placement(0, 0, P, None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_placement(4097, 0, P, None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_placement(256, 0, P + 2, None) == B.STATUS["ALIGNMENT"]
-    res = B.ProbeHandoverResult()
-    assert lib.llmi_hip_probe_handover(5, 2, 0, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 0, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 0, 16, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
-    assert lib.llmi_hip_probe_handover(0, 2, 3, 8, 0, P + 16, ctypes.byref(res), None) == B.STATUS["ALIGNMENT"]
+    diag = B.diag_lib()
+    assert diag.llmi_diag_handover(0, 2, 0, 8, 0, None, None, None) == B.STATUS["NULL_POINTER"]
+    assert diag.llmi_diag_placement(256, 0, None, None) == B.STATUS["NULL_POINTER"]
+    assert diag.llmi_diag_placement(0, 0, P, None) == B.STATUS["INVALID_ARG"]
+    assert diag.llmi_diag_placement(4097, 0, P, None) == B.STATUS["INVALID_ARG"]
+    assert diag.llmi_diag_placement(256, 0, P + 2, None) == B.STATUS["ALIGNMENT"]
+    res = B.DiagHandoverResult()
+    assert diag.llmi_diag_handover(5, 2, 0, 8, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert diag.llmi_diag_handover(0, 2, 0, 0, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert diag.llmi_diag_handover(0, 2, 0, 16, 0, P, ctypes.byref(res), None) == B.STATUS["INVALID_ARG"]
+    assert diag.llmi_diag_handover(0, 2, 3, 8, 0, P + 16, ctypes.byref(res), None) == B.STATUS["ALIGNMENT"]
 
 
 @pytest.fixture(scope="module")
@@ -103,7 +105,7 @@ def test_handover_probe_device_scope_sees_the_store(dev, reader):
     line = torch.zeros(4096 // 4 + 64, dtype=torch.int32, device=dev)
     base = (line.data_ptr() + 255) & ~255
     res = torch.zeros(8, dtype=torch.int32, device=dev)
-    rc = B.lib().llmi_hip_probe_handover(B.PROBE_SC1, B.PROBE_SC1, 0, reader, 1, base, res.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    rc = B.diag_lib().llmi_diag_handover(B.DIAG_SC1, B.DIAG_SC1, 0, reader, 1, base, res.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     seen, polls, ns, xr, xw = (int(x) for x in res[:5].cpu())
@@ -114,25 +116,25 @@ def test_handover_probe_device_scope_sees_the_store(dev, reader):
 @pytest.mark.gpu
 @pytest.mark.parametrize("exclusive", [0, 1])
 def test_placement_probe_names_a_cu_for_every_workgroup(dev, exclusive):
-    """One workgroup per CU is what the split path's grid counts on: 256 workgroups with a decode workgroup's LDS
-    footprint report their XCD and CU; every XCD takes its share and at least half the grid has a CU of its own
-    (on the boxes measured: all 256)."""
+    """256 workgroups with a decode workgroup's LDS footprint report their XCD and CU (on the boxes measured: 256
+    different CUs, 32 per XCD; printed, not asserted: the split path does not rely on it for its result)."""
     import torch
     ids = torch.zeros(2 * 256, dtype=torch.int32, device=dev)
-    assert B.lib().llmi_hip_probe_placement(256, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    assert B.diag_lib().llmi_diag_placement(256, exclusive, ids.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
     torch.cuda.synchronize()
     a = ids.cpu().numpy().astype(np.uint32).reshape(-1, 2)
     assert np.all(a[:, 0] < 16) and np.all(a[:, 1] != 0)
     cus = {(int(x), (int(h) >> 8) & 0xFF) for x, h in a}
-    assert len(cus) >= 128
-    assert len(set(int(x) for x in a[:, 0])) >= 1
+    print("placement: %d distinct CUs, %d XCDs for 256 workgroups" % (len(cus), len(set(int(x) for x in a[:, 0]))))
 
 
 @pytest.mark.gpu
 def test_pingpong_probe_times_both_blocks_from_every_xcd(dev):
     """Eight pairs of workgroups, each pair on one XCD, hand 64 numbers to and fro through two neighbouring 8 KiB blocks:
-    every number arrives, the pairs cover both sides of the package, the times are a few hundred ns per hand-over, and
-    the two sides disagree about which block is nearer (what llmi_hip_mha_workspace_side reads off)."""
+    every number arrives and every workgroup names the XCD it ran on (pairs share one when workgroups are dealt to the
+    XCDs in turn; a pair that did not is left out of the decision). The times (a few hundred ns per hand-over on the boxes measured,
+    the two sides of the package disagreeing about which block is nearer) are what llmi_hip_mha_workspace_side reads
+    off; they are printed here, the decision taken from them is tested with made-up timings on the CPU."""
     import torch
     buf = torch.zeros((64 << 10) // 4, dtype=torch.int32, device=dev)
     base = (buf.data_ptr() + 16383) & ~16383
@@ -141,9 +143,10 @@ def test_pingpong_probe_times_both_blocks_from_every_xcd(dev):
     torch.cuda.synchronize()
     r = out.cpu().numpy().astype(np.int64).reshape(8, 8)
     assert np.all(r[:, 3] == 1)                                   # nothing lost
-    assert np.all(r[:, 0] == r[:, 5]) and np.all(r[:, 0] < 8)     # a pair shares an XCD
-    assert {int(x) >> 2 for x in r[:, 0]} == {0, 1}               # both sides of the package
+    assert np.all(r[:, 0] < 8) and np.all(r[:, 5] < 8)            # both workgroups of a pair name their XCD
+    assert np.all(r[:, 1:3] > 0)
     per_handover_ns = r[:, 1:3] * 10 / 64
-    assert np.all(per_handover_ns > 100) and np.all(per_handover_ns < 5000)
-    d = [np.mean((r[:, 1] - r[:, 2])[(r[:, 0] >> 2) == s]) for s in (0, 1)]
-    assert d[0] * d[1] < 0
+    d = [np.mean((r[:, 1] - r[:, 2])[(r[:, 0] >> 2) == s]) if np.any((r[:, 0] >> 2) == s) else float("nan") for s in (0, 1)]
+    print("ping-pong: %d of 8 pairs on one XCD; %.0f .. %.0f ns per hand-over; clear minus set block, ticks: XCDs 0-3 %+.0f, XCDs 4-7 %+.0f; decision %d"
+          % (int(np.sum(r[:, 0] == r[:, 5])), per_handover_ns.min(), per_handover_ns.max(), d[0], d[1],
+             B.lib().llmi_hip_side_from_pingpong(out.cpu().numpy().astype(np.uint32).ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))))
