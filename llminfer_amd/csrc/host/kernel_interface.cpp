@@ -22,8 +22,23 @@ void mha_kernel_hip_slot(const tensor::Tensor& query, const tensor::Tensor& key_
 }
 }  // namespace
 
+// The library this layer was linked against must speak the ABI of the header it was compiled with: a struct that
+// grew since would be read past its end. Checked once, the first time a HIP arm is handed out.
+static void ensure_abi() {
+    static const bool ok = [] {
+        const int got = llmi_hip_abi_version();
+        if (got != LLMI_HIP_ABI_VERSION)
+            LLMI_FATAL("libllmi_hip.so speaks ABI version " << got << ", this host layer was built for " << LLMI_HIP_ABI_VERSION);
+        return true;
+    }();
+    (void)ok;
+}
+
 MHAKernel get_mha_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return mha_kernel_hip_slot;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return mha_kernel_hip_slot;
+    }
     if (device_type == base::DeviceType::DeviceCPU && g_cpu_mha) return g_cpu_mha;
     LLMI_FATAL("Unknown device type for get a mha kernel.");
 }
@@ -34,27 +49,42 @@ void register_mha_kernel(base::DeviceType device_type, MHAKernel fn) {
 }
 
 FusedQKNormRoPEKernel get_fused_qk_norm_rope_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return fused_qk_norm_rope_kernel_hip;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return fused_qk_norm_rope_kernel_hip;
+    }
     LLMI_FATAL("Unknown device type for get a fused_qk_norm_rope kernel.");  // kernel_interface.cpp:172-178: GPU only
 }
 
 SinCosCacheKernel get_sin_cos_cache_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return sin_cos_cache_precompute_hip;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return sin_cos_cache_precompute_hip;
+    }
     LLMI_FATAL("Unknown device type for get a sin_cos_cache kernel.");
 }
 
 GEMVKernel get_gemv_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return gemv_kernel_hip;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return gemv_kernel_hip;
+    }
     LLMI_FATAL("Unknown device type for get a gemv kernel.");
 }
 
 FusedGEMVAddKernel get_fused_gemv_add_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return fused_gemv_add_kernel_hip;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return fused_gemv_add_kernel_hip;
+    }
     LLMI_FATAL("Unknown device type for get a fused_gemv_add kernel.");
 }
 
 FusedQKVGEMVKernel get_fused_qkv_gemv_kernel(base::DeviceType device_type) {
-    if (device_type == base::DeviceType::DeviceHIP) return fused_qkv_gemv_kernel_hip;
+    if (device_type == base::DeviceType::DeviceHIP) {
+        ensure_abi();
+        return fused_qkv_gemv_kernel_hip;
+    }
     LLMI_FATAL("Unknown device type for get a fused_qkv_gemv kernel.");
 }
 
