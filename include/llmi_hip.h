@@ -15,6 +15,8 @@
  *                                 code/source/op/mha.cpp:54-56)
  *   llmi_hip_mha_decode_append    the pair fused_qk_norm_rope_kernel_cu + mha_kernel_cu as
  *                                 the layer loop issues it, code/source/model/qwen3_fused.cpp:524-548
+ *   llmi_hip_mha_decode_append_stack  that pair for every layer of the layer loop,
+ *                                 code/source/model/qwen3_fused.cpp:115-127 (one resident launch)
  *   llmi_hip_mha_workspace_bytes  the KVSplitOutput buffer sizing
  *                                 code/source/model/qwen3_fused.cpp:502-503
  *   llmi_hip_mha_plan             the dispatch arithmetic inside mha_kernel_cu
@@ -48,7 +50,8 @@ extern "C" {
 
 /* Bumped whenever a struct below changes size or layout, or an entry point changes meaning: a caller compiled
  * against another value must not call into this library (llmi_hip_abi_version() returns the library's).
- * 3: llmi_mha_args.workspace_side, llmi_mha_plan.workspace_side, llmi_attn_oproj_args.one_launch. */
+ * 3: llmi_mha_args.workspace_side, llmi_mha_plan.workspace_side, llmi_attn_oproj_args.one_launch,
+ *    llmi_hip_mha_decode_append_stack. */
 #define LLMI_HIP_ABI_VERSION 3
 
 typedef enum llmi_status {
@@ -200,6 +203,38 @@ typedef struct llmi_attn_oproj_args {
  * llmi_hip_mha_oproj_launches tells which: 1 or 2 (or a negative status for invalid arguments). */
 int llmi_hip_mha_decode_append_oproj(const llmi_attn_oproj_args* args);
 int llmi_hip_mha_oproj_launches(const llmi_attn_oproj_args* args);
+
+typedef struct llmi_mha_stack_args {
+    llmi_mha_append_args first; /* the first layer's call, exactly as for llmi_hip_mha_decode_append
+                                   (first.mha.layer_id = the first layer of the run)                                  */
+    int32_t layer_count;        /* consecutive layers, >= 1; layer l of the run uses cache layer first.mha.layer_id + l */
+    /* elements (bf16) between one layer's buffer and the next layer's; multiples of 8; 0 = every layer uses the same */
+    int64_t query_stride;       /* first.mha.query      + l * query_stride       = layer l's raw query [head_num*128]  */
+    int64_t key_new_stride;     /* first.key_new        + l * key_new_stride     = layer l's raw K row [kv_dim]        */
+    int64_t value_new_stride;   /* first.value_new      + l * value_new_stride   = layer l's V row [kv_dim]            */
+    int64_t norm_weight_stride; /* first.norm_weight    + l * norm_weight_stride = layer l's q_norm | k_norm [2*128]   */
+    int64_t output_stride;      /* first.mha.output     + l * output_stride      = layer l's output [head_num*128]
+                                   (and first.mha.output_f32 + l * output_stride, in floats, if that tap is set)       */
+} llmi_mha_stack_args;
+
+/* llmi_hip_mha_decode_append for `layer_count` consecutive layers at one position, in layer order: the attention part
+ * of one decode step as the reference's layer loop issues it (code/source/model/qwen3_fused.cpp:115-127: per layer
+ * fused_qk_norm_rope + mha, :524-548). Same results as that many calls, bit for bit, including when buffers alias
+ * across layers (a layer's query may be the previous layer's output: a layer reads its query, K row and V row only
+ * after the previous layer's output is complete).
+ * Where the shape allows it this is ONE launch: the split path's grid stays resident and walks the layers itself, every
+ * wavefront streaming its K/V tiles of all layers as one sequence (the next layer's tiles are on their way while this
+ * layer's partial results are handed over and merged), and a layer's inputs are read only after every query head of
+ * the layer before has published a "done" tag behind its acknowledged output. Workgroups wait for other workgroups of
+ * the same launch there, so every workgroup of the grid has to be resident at once: call this only on a GPU that runs
+ * nothing else at the time. Every wait is bounded (llmi_hip_set_poll_limit); one that gives up is counted
+ * (llmi_hip_poll_timeouts) and turns the outputs of its layer and the following ones into NaN. The one-launch form
+ * needs: the fused split path with 2..64 splits and a host-side position, a query group of at most 4 heads, a grid no
+ * larger than the device's compute unit count, and a workspace sized by llmi_hip_mha_workspace_bytes (the plan's need
+ * plus 4.3 KiB for the tags). Anything else runs as layer_count launches of llmi_hip_mha_decode_append.
+ * llmi_hip_mha_stack_launches tells which: 1 or layer_count (or a negative status for invalid arguments). */
+int llmi_hip_mha_decode_append_stack(const llmi_mha_stack_args* args);
+int llmi_hip_mha_stack_launches(const llmi_mha_stack_args* args);
 
 /* Bytes of fp32 workspace that are enough for any pos < max_seq_len. */
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len);

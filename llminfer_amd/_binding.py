@@ -46,6 +46,12 @@ class AttnOprojArgs(ctypes.Structure):
     _fields_ = [("attn", MhaAppendArgs), ("o_weight", c_void_p), ("residual", c_void_p), ("hidden", c_i32), ("one_launch", c_i32)]
 
 
+class MhaStackArgs(ctypes.Structure):
+    _fields_ = [("first", MhaAppendArgs), ("layer_count", c_i32), ("query_stride", ctypes.c_int64),
+                ("key_new_stride", ctypes.c_int64), ("value_new_stride", ctypes.c_int64),
+                ("norm_weight_stride", ctypes.c_int64), ("output_stride", ctypes.c_int64)]
+
+
 class GemvArgs(ctypes.Structure):
     _fields_ = [
         ("input", c_void_p), ("weight", c_void_p), ("output", c_void_p),
@@ -106,6 +112,8 @@ SYMBOLS = {
     "llmi_hip_mha_decode_append": (ctypes.c_int, [ctypes.POINTER(MhaAppendArgs)]),
     "llmi_hip_mha_decode_append_oproj": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
     "llmi_hip_mha_oproj_launches": (ctypes.c_int, [ctypes.POINTER(AttnOprojArgs)]),
+    "llmi_hip_mha_decode_append_stack": (ctypes.c_int, [ctypes.POINTER(MhaStackArgs)]),
+    "llmi_hip_mha_stack_launches": (ctypes.c_int, [ctypes.POINTER(MhaStackArgs)]),
     "llmi_hip_mha_workspace_bytes": (c_size_t, [c_i32, c_i32, c_i32]),
     "llmi_hip_mha_workspace_side": (ctypes.c_int, [c_void_p, c_size_t, c_void_p, ctypes.POINTER(c_i32)]),
     "llmi_hip_qk_norm_rope_append": (ctypes.c_int, [ctypes.POINTER(QkNormRopeArgs)]),

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(HERE, "libllmi_hip.so")
 HOST_LIB_PATH = os.path.join(HERE, "libllmi_host.so")
 DIAG_LIB_PATH = os.path.join(HERE, "libllmi_diag.so")
 
-HIP_SOURCES = ["mha_decode_group4.hip", "mha_decode_group8.hip", "mha_decode_group16.hip", "mha_decode_group2.hip", "mha_decode_group1.hip",
+HIP_SOURCES = ["mha_decode_group4.hip", "mha_decode_group8.hip", "mha_decode_group16.hip", "mha_decode_group2.hip", "mha_decode_group1.hip", "mha_stack.hip",
                "mha_decode.hip", "qk_norm_rope.hip", "gemv.hip", "probes.hip", "c_api.cpp", "pool.cpp"]
 DIAG_SOURCES = ["diag_probes.hip"]
 

@@ -91,8 +91,18 @@ unsigned long long next_epoch() {
     return counter.fetch_add(1, std::memory_order_relaxed);
 }
 
-// Default: far beyond any real kernel time (seconds), yet finite.
-static std::atomic<int> g_poll_limit{1 << 22};
+// Default: far beyond any real kernel time (seconds), yet finite. LLMI_HIP_POLL_LIMIT in the environment replaces the
+// default (read once, when the library is loaded); llmi_hip_set_poll_limit changes it at run time.
+static int default_poll_limit() {
+    const char* v = std::getenv("LLMI_HIP_POLL_LIMIT");
+    if (v && *v) {
+        char* end = nullptr;
+        const long x = std::strtol(v, &end, 10);
+        if (end && *end == '\0' && x >= 0 && x <= INT32_MAX) return (int)x;
+    }
+    return 1 << 22;
+}
+static std::atomic<int> g_poll_limit{default_poll_limit()};
 int poll_limit() { return g_poll_limit.load(std::memory_order_relaxed); }
 static std::atomic<int> g_test_far_home{0};
 int test_far_home() { return g_test_far_home.load(std::memory_order_relaxed); }
@@ -332,6 +342,21 @@ int llmi_hip_mha_decode_append(const llmi_mha_append_args* args) {
     return launch_mha_decode(args->mha, plan, args);
 }
 
+// Compute units of the current device (asked once per process), or 0 if the device cannot be asked.
+static int compute_units() {
+    static std::atomic<int> cu_count{0};
+    int cus = cu_count.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        cu_count.store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 // Validates the arguments and decides between the one-launch form (*fused = true, plan filled) and the pair.
 static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, bool* fused) {
     if (!args) return LLMI_ERR_NULL_POINTER;
@@ -354,16 +379,8 @@ static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, boo
     const int64_t k = (int64_t)m.head_num * m.head_dim;
     if (m.pos_device || k % 512 != 0 || k > max_k || m.head_num > 128) return LLMI_OK;  // (one wavefront collects the heads' tags, two per lane)
     // every workgroup must be resident at once: the workers wait for the combiners
-    static std::atomic<int> cu_count{0};
-    int cus = cu_count.load(std::memory_order_relaxed);
-    if (cus == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
-            (void)hipGetLastError();
-            return LLMI_OK;
-        }
-        cu_count.store(cus, std::memory_order_relaxed);
-    }
+    const int cus = compute_units();
+    if (cus <= 0) return LLMI_OK;
     auto fits = [&](const llmi_mha_plan& p) {
         if (p.path != LLMI_PATH_SPLIT_FUSED || p.num_splits < 2) return false;
         if (p.group_pad > 8 || p.waves_per_group != (p.group_pad == 8 ? 8 : 4)) return false;
@@ -411,6 +428,62 @@ int llmi_hip_mha_decode_append_oproj(const llmi_attn_oproj_args* args) {
                        static_cast<hipStream_t>(m.stream));
 }
 
+// Validates a multi-layer call and decides between the one-launch form (*one_launch = true, plan = layer 0's) and
+// one launch per layer.
+static int plan_stack(const llmi_mha_stack_args* args, llmi_mha_plan* plan, bool* one_launch) {
+    if (!args) return LLMI_ERR_NULL_POINTER;
+    const llmi_mha_append_args& ap = args->first;
+    if (!ap.key_new || !ap.value_new || !ap.norm_weight || !ap.sin_cache || !ap.cos_cache) return LLMI_ERR_NULL_POINTER;
+    const void* ptrs[] = {ap.key_new, ap.value_new, ap.norm_weight, ap.sin_cache, ap.cos_cache};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return LLMI_ERR_ALIGNMENT;
+    if (!(ap.eps >= 0.0f) || args->layer_count < 1) return LLMI_ERR_INVALID_ARG;
+    if (ap.mha.force_path == LLMI_PATH_SPLIT) return LLMI_ERR_INVALID_ARG;
+    const int64_t strides[] = {args->query_stride, args->key_new_stride, args->value_new_stride, args->norm_weight_stride,
+                               args->output_stride};
+    for (int64_t st : strides)
+        if (st % 8 != 0) return LLMI_ERR_ALIGNMENT;  // (every layer's rows stay 16-byte aligned)
+    if ((int64_t)ap.mha.layer_id + args->layer_count > INT32_MAX) return LLMI_ERR_INVALID_ARG;
+    if (int rc = make_plan(&ap.mha, plan, kMaxWaves, 1)) return rc;
+    *one_launch = false;
+    const llmi_mha_args& m = ap.mha;
+    if (m.pos_device) return LLMI_OK;
+    if (plan->path != LLMI_PATH_SPLIT_FUSED || plan->num_splits < 2 || plan->num_splits > 64) return LLMI_OK;
+    if (plan->group_pad > 4 || plan->waves_per_group != 4) return LLMI_OK;
+    if (m.workspace_bytes < plan->workspace_needed + stack_workspace_extra(m.head_num)) return LLMI_OK;
+    // every workgroup must be resident at once: workgroups wait for each other
+    const int cus = compute_units();
+    if (cus <= 0 || (int64_t)(m.kv_dim / m.head_dim) * plan->num_splits > cus) return LLMI_OK;
+    *one_launch = true;
+    return LLMI_OK;
+}
+
+int llmi_hip_mha_stack_launches(const llmi_mha_stack_args* args) {
+    llmi_mha_plan plan;
+    bool one = false;
+    if (int rc = plan_stack(args, &plan, &one)) return rc;
+    return one ? 1 : args->layer_count;
+}
+
+int llmi_hip_mha_decode_append_stack(const llmi_mha_stack_args* args) {
+    llmi_mha_plan plan;
+    bool one = false;
+    if (int rc = plan_stack(args, &plan, &one)) return rc;
+    if (one) return launch_mha_stack(*args, plan);
+    for (int32_t l = 0; l < args->layer_count; ++l) {
+        llmi_mha_append_args a = args->first;
+        a.mha.layer_id += l;
+        a.mha.query = static_cast<const uint16_t*>(a.mha.query) + l * args->query_stride;
+        a.key_new = static_cast<const uint16_t*>(a.key_new) + l * args->key_new_stride;
+        a.value_new = static_cast<const uint16_t*>(a.value_new) + l * args->value_new_stride;
+        a.norm_weight = static_cast<const uint16_t*>(a.norm_weight) + l * args->norm_weight_stride;
+        a.mha.output = static_cast<uint16_t*>(a.mha.output) + l * args->output_stride;
+        if (a.mha.output_f32) a.mha.output_f32 += l * args->output_stride;
+        if (int rc = launch_mha_decode(a.mha, plan, &a)) return rc;
+    }
+    return LLMI_OK;
+}
+
 size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t max_seq_len) {
     if (head_num <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
     int splits = (max_seq_len + kTile - 1) / kTile;
@@ -423,7 +496,8 @@ size_t llmi_hip_mha_workspace_bytes(int32_t head_num, int32_t head_dim, int32_t 
     const size_t plain = (size_t)head_num * (size_t)splits * ((size_t)head_dim * sizeof(float) + 2 * sizeof(unsigned long long)) + 16;
     // (the layout by side exists for the head_dim the kernels take; a row of any other width would not fit its 8 KiB blocks)
     const size_t by_side = head_dim == 128 ? fused_workspace(head_num, head_dim, splits, true).bytes() + 2 * kSideBlock : 0;
-    size_t need = (plain > by_side ? plain : by_side) + (size_t)head_num * sizeof(uint32_t);
+    // ... and the multi-layer launch's done tags
+    size_t need = (plain > by_side ? plain : by_side) + (size_t)head_num * sizeof(uint32_t) + stack_workspace_extra(head_num);
     if (need < 6 * kSideBlock) need = 6 * kSideBlock;
     return need;
 }

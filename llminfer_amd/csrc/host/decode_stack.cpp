@@ -90,6 +90,46 @@ void DecodeStack::enqueue(int32_t pos, int32_t mode, bool follow_device_pos) {
     tensor::Tensor& vc = buffers_->get_buffer(ModelBufferType::ValueCache);
     tensor::Tensor& q = buffers_->get_buffer(ModelBufferType::Query);
     tensor::Tensor& ws = buffers_->get_buffer(ModelBufferType::KVSplitOutput);
+    if (mode == kResidentStack) {
+        LLMI_CHECK(!follow_device_pos);
+        llmi_mha_stack_args t{};
+        llmi_mha_args& m = t.first.mha;
+        m.query = query_raw(0);
+        m.key_cache = kc.ptr<uint16_t>();
+        m.value_cache = vc.ptr<uint16_t>();
+        m.workspace = ws.ptr<float>();
+        m.workspace_bytes = ws.byte_size();
+        m.output = output(0);
+        m.layer_id = 0;
+        m.pos = pos;
+        m.kv_dim = c.kv_dim();
+        m.kv_mul = c.kv_mul();
+        m.head_num = c.head_num;
+        m.head_dim = c.head_dim;
+        m.max_seq_len = c.max_seq_len;
+        m.kv_layout = c.kv_layout;
+        const kernel::MhaHipOptions& o = kernel::mha_hip_options();
+        m.force_path = o.force_path;
+        m.num_splits = o.num_splits;
+        m.waves_per_group = o.waves_per_group;
+        m.stream = stream();
+        m.workspace_side = kernel::workspace_side_of(m.workspace, m.workspace_bytes, stream());
+        t.first.key_new = key_raw(0);
+        t.first.value_new = value_raw(0);
+        t.first.norm_weight = norm_weight(0);
+        t.first.sin_cache = buffers_->get_buffer(ModelBufferType::SinCache).ptr<float>();
+        t.first.cos_cache = buffers_->get_buffer(ModelBufferType::CosCache).ptr<float>();
+        t.first.eps = 1e-6f;
+        t.layer_count = c.layer_num;
+        t.query_stride = c.dim();
+        t.key_new_stride = c.kv_dim();
+        t.value_new_stride = c.kv_dim();
+        t.norm_weight_stride = 2 * c.head_dim;
+        t.output_stride = c.dim();
+        const int rc = llmi_hip_mha_decode_append_stack(&t);
+        if (rc != LLMI_OK) LLMI_FATAL("llmi_hip_mha_decode_append_stack: " << llmi_hip_strerror(rc) << " " << llmi_hip_last_error());
+        return;
+    }
     for (int32_t layer = 0; layer < c.layer_num; ++layer) {
         const void* q_for_attention = query_raw(layer);
         if (with_qk_norm_rope) {

@@ -56,7 +56,11 @@ public:
     // three launches per layer.
     // kFusedBlock (4): the same block in two launches per layer: packed QKV GEMV -> attention whose idle
     // workgroups also do the output projection + residual (llmi_hip_mha_decode_append_oproj).
-    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2, kAttentionBlock = 3, kFusedBlock = 4 };
+    // kResidentStack (5): what kFusedAppend computes, as ONE launch for all layers (llmi_hip_mha_decode_append_stack):
+    // the grid stays resident, the next layer's K/V tiles are on their way while this layer's results are merged,
+    // and a layer reads its inputs only after the layer before has published its outputs.
+    enum Mode : int32_t { kAttentionOnly = 0, kSeparateQkNormRope = 1, kFusedAppend = 2, kAttentionBlock = 3, kFusedBlock = 4,
+                          kResidentStack = 5 };
     // Enqueues the whole stack for a token at `pos` on the stack's stream (no synchronisation).
     // `follow_device_pos`: the kernels read the position from the stack's device word (set_position)
     // and `pos` is the largest position they may see; modes 0 and 2 only (the separate QK-Norm/RoPE

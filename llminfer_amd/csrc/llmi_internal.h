@@ -75,6 +75,10 @@ int test_far_home();
 // `oproj` non-null (with `append`): the attention launch also computes the output projection + residual add.
 int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append = nullptr,
                       const llmi_attn_oproj_args* oproj = nullptr);
+// The multi-layer launch (llmi_hip_mha_decode_append_stack in its one-launch form); `plan` is layer 0's.
+int launch_mha_stack(const llmi_mha_stack_args& st, const llmi_mha_plan& plan);
+// Bytes the multi-layer launch keeps behind the fused combine's records (its "done" tags, with room to align them).
+size_t stack_workspace_extra(int head_num);
 // What the fused projection holds per wavefront: weight rows, and the widest attention output (elements).
 int oproj_limits(int32_t* rows_per_wave, int32_t* max_k);
 int launch_qk_norm_rope_append(const llmi_qk_norm_rope_args& args);

@@ -109,7 +109,7 @@ int static_scratch(void** ptr, size_t* bytes) {
 int read_poll_timeouts(unsigned long long* count) {
     // (every translation unit that instantiates the kernels counts on its own device word)
     hipError_t (*const parts[])(unsigned int*) = {poll_timeouts_group1, poll_timeouts_group2, poll_timeouts_group4,
-                                                  poll_timeouts_group8, poll_timeouts_group16};
+                                                  poll_timeouts_group8, poll_timeouts_group16, poll_timeouts_stack};
     unsigned long long total = 0;
     for (auto part : parts) {
         unsigned int n = 0;
@@ -120,9 +120,10 @@ int read_poll_timeouts(unsigned long long* count) {
     return LLMI_OK;
 }
 
-int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append,
-                      const llmi_attn_oproj_args* oproj) {
-    const int n_kv = args.kv_dim / args.head_dim;
+// The kernels' argument block for one call. *fused_end: the first byte behind the fused combine's records in the
+// workspace (where the one-launch projection and the multi-layer kernel keep their words), or nullptr.
+static int fill_kernel_args(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append,
+                            const llmi_attn_oproj_args* oproj, int tags, KernelArgs* out_ka, char** out_fused_end) {
     const int64_t layer_off = (int64_t)args.layer_id * args.max_seq_len * args.kv_dim;
 
     KernelArgs ka{};
@@ -168,7 +169,10 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         }
         ka.records = reinterpret_cast<unsigned long long*>(base + fw.partial_bytes);
         fused_end = base + fw.partial_bytes + fw.record_bytes;
-        ka.tag = record_tag(next_epoch());
+        // (a multi-layer launch takes one tag per layer, consecutive ones)
+        const unsigned long long epoch = next_epoch();
+        for (int i = 1; i < tags; ++i) (void)next_epoch();
+        ka.tag = record_tag(epoch);
     }
     if (args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) {
         ka.row_stride = args.kv_dim;
@@ -206,6 +210,38 @@ int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, cons
         ka.o_res = static_cast<uint16_t*>(oproj->residual);
         ka.o_n = oproj->hidden;
     }
+    *out_ka = ka;
+    if (out_fused_end) *out_fused_end = fused_end;
+    return LLMI_OK;
+}
+
+size_t stack_workspace_extra(int head_num) { return 256 + stack_done_bytes(head_num); }
+
+int launch_mha_stack(const llmi_mha_stack_args& st, const llmi_mha_plan& plan) {
+    const llmi_mha_args& m = st.first.mha;
+    StackArgs sa{};
+    char* fused_end = nullptr;
+    if (int rc = fill_kernel_args(m, plan, &st.first, nullptr, st.layer_count, &sa.a, &fused_end)) return rc;
+    if (!fused_end) return LLMI_ERR_INVALID_ARG;  // (the caller has checked: fused split path)
+    sa.layers = st.layer_count;
+    sa.q_stride = st.query_stride;
+    sa.knew_stride = st.key_new_stride;
+    sa.vnew_stride = st.value_new_stride;
+    sa.normw_stride = st.norm_weight_stride;
+    sa.out_stride = st.output_stride;
+    sa.cache_stride = (int64_t)m.max_seq_len * m.kv_dim;
+    // the heads' done tags: behind the records, on a 256-byte line of their own
+    sa.done = reinterpret_cast<uint32_t*>((reinterpret_cast<uintptr_t>(fused_end) + 255u) & ~(uintptr_t)255u);
+    if (!launch_stack(sa, m.kv_dim / m.head_dim, plan.group_pad, plan.waves_per_group, static_cast<hipStream_t>(m.stream)))
+        return LLMI_ERR_INVALID_ARG;
+    return check_launch();
+}
+
+int launch_mha_decode(const llmi_mha_args& args, const llmi_mha_plan& plan, const llmi_mha_append_args* append,
+                      const llmi_attn_oproj_args* oproj) {
+    const int n_kv = args.kv_dim / args.head_dim;
+    KernelArgs ka{};
+    if (int rc = fill_kernel_args(args, plan, append, oproj, 1, &ka, nullptr)) return rc;
 
     hipStream_t stream = static_cast<hipStream_t>(args.stream);
     const bool ap = append != nullptr;

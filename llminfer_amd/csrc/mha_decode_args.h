@@ -53,6 +53,20 @@ struct KernelArgs {
     int32_t far_home;  // testing aid: 1 = every split but the merging one, 2 = every second one uses the other side's home
 };
 
+// The multi-layer kernel (mha_stack.hip): `a` holds layer 0's arguments; layer l uses the same ones with the pointers
+// moved on by l strides (elements) and the record tag a.tag + l.
+struct StackArgs {
+    KernelArgs a;
+    int32_t layers;
+    int64_t q_stride, knew_stride, vnew_stride, normw_stride, out_stride;  // elements between consecutive layers
+    int64_t cache_stride;  // elements between consecutive layers' K (and V) caches
+    uint32_t* done;        // in the workspace: the heads' "done" tags, stack_done_bytes() bytes
+};
+// Groups of 1, 2 or 4 query heads (padded), four wavefronts per workgroup; false otherwise.
+bool launch_stack(const StackArgs& sa, int n_kv, int group_pad, int waves, hipStream_t stream);
+size_t stack_done_bytes(int head_num);
+hipError_t poll_timeouts_stack(unsigned int* n);
+
 // Launchers of the kernels instantiated for a (padded) group of G query heads per KV head; each lives in its own
 // translation unit so that the groups compile side by side. `nw`: wavefronts per workgroup; false if the kernel is
 // not instantiated for that count.

@@ -147,6 +147,31 @@ def mha_decode_append(query_raw, key_new, value_new, norm_weight, sin_cache, cos
     return launches
 
 
+def mha_decode_append_stack(query_raw, key_new, value_new, norm_weight, sin_cache, cos_cache, key_cache, value_cache,
+                            output, workspace, *, layer_count, query_stride, key_new_stride, value_new_stride,
+                            norm_weight_stride, output_stride, eps=1e-6, stream=None, **kw):
+    """llmi_hip_mha_decode_append for `layer_count` consecutive layers (llmi_hip_mha_decode_append_stack): the tensors
+    are the first layer's, layer l uses them moved on by l strides (elements). Returns the launch count."""
+    for name, t in (("query_raw", query_raw), ("key_new", key_new), ("value_new", value_new),
+                    ("norm_weight", norm_weight), ("key_cache", key_cache), ("value_cache", value_cache),
+                    ("output", output)):
+        _check_dev(name, t, _BF16_DTYPES)
+    for name, t in (("sin_cache", sin_cache), ("cos_cache", cos_cache), ("workspace", workspace),
+                    ("output_f32", kw.get("output_f32"))):
+        _check_dev(name, t, (torch.float32,))
+    t = B.MhaStackArgs()
+    a = t.first
+    a.mha = make_mha_args(query_raw, key_cache, value_cache, output, workspace, stream=_stream_handle(stream), **kw)
+    a.key_new, a.value_new, a.norm_weight = _ptr(key_new), _ptr(value_new), _ptr(norm_weight)
+    a.sin_cache, a.cos_cache, a.eps = _ptr(sin_cache), _ptr(cos_cache), eps
+    t.layer_count = layer_count
+    t.query_stride, t.key_new_stride, t.value_new_stride = query_stride, key_new_stride, value_new_stride
+    t.norm_weight_stride, t.output_stride = norm_weight_stride, output_stride
+    launches = B.lib().llmi_hip_mha_stack_launches(ctypes.byref(t))
+    B.check(B.lib().llmi_hip_mha_decode_append_stack(ctypes.byref(t)), "llmi_hip_mha_decode_append_stack")
+    return launches
+
+
 def sincos_table(head_dim, max_seq_len, device="cuda", stream=None):
     sin = torch.empty((max_seq_len, head_dim // 2), dtype=torch.float32, device=device)
     cos = torch.empty_like(sin)

@@ -332,6 +332,30 @@ def test_decode_stack_eager_and_graph_match_oracle(oracle, dev, layout, layers, 
             check("replay %d" % rep)
             torch.randn(1000, device=dev).sum().item()  # eager work between replays
         assert ms.value > 0
+        # the same step as ONE resident launch for all layers (mode 5): the bits of mode 2, eager and replayed
+        want = [_download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16) for l in range(layers)]
+
+        def check_bits(tag):
+            for l in range(layers):
+                got = _download(H.L.llmi_host_stack_ptr(stack, 6, l), (n_q * d,), np.uint16)
+                assert np.array_equal(got, want[l]), "%s layer %d" % (tag, l)
+
+        def wipe():
+            _upload(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up)
+            _upload(H.L.llmi_host_stack_ptr(stack, 1, 0), v_up)
+            for l in range(layers):
+                _upload(H.L.llmi_host_stack_ptr(stack, 6, l), np.zeros(n_q * d, dtype=np.uint16))
+
+        wipe()
+        H.ok(H.L.llmi_host_stack_run(stack, pos, 5))
+        check_bits("resident, eager")
+        assert np.array_equal(_download(H.L.llmi_host_stack_ptr(stack, 0, 0), k_up.shape, np.uint16), k_fused)
+        H.ok(H.L.llmi_host_stack_capture(stack, pos, 5))
+        for rep in range(3):
+            wipe()
+            H.ok(H.L.llmi_host_stack_replay(stack, 1, ctypes.byref(ms)))
+            check_bits("resident, replay %d" % rep)
+            torch.randn(1000, device=dev).sum().item()
     finally:
         H.L.llmi_host_stack_destroy(stack)
 
