@@ -301,9 +301,13 @@ def stack_result(args, ctx):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(us_token / 1e3, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%d layers x (fused QK-Norm + RoPE + K/V append, GQA decode attention), %d Q / 8 KV "
-                               "heads, ctx %d + 1 new token, one HIP graph per token, %s layout, %s"
-                               % (layers, n_q, ctx, "head-major" if args.layout == 1 else "position-major",
+                               "heads, ctx %d + 1 new token, %d per-layer caches (one random cache rolled per layer: distinct "
+                               "addresses and values, 604 MB walked per token at 36 layers), one HIP graph per token, %s layout, %s"
+                               % (layers, n_q, ctx, layers, "head-major" if args.layout == 1 else "position-major",
                                   "one launch per layer" if args.stack_mode == 2 else
+                                  "ONE resident launch for all layers (llmi_hip_mha_decode_append_stack): the next layer's K/V tiles "
+                                  "stream while this layer's results are merged, and a layer reads its query / K row / V row only after "
+                                  "every head of the layer before has published its output" if args.stack_mode == 5 else
                                   "three launches per layer: packed QKV GEMV (hidden %d), attention, output projection + "
                                   "residual" % hidden if args.stack_mode == 3 else
                                   "two launches per layer: packed QKV GEMV (hidden %d), attention whose idle workgroups do the "
@@ -569,7 +573,7 @@ def main():
     ap.add_argument("--stack-follow-pos", action="store_true",
                     help="with --stack: capture once for every position (kernels read it from device memory)")
     ap.add_argument("--stack-mode", type=int, default=2,
-                    help="with --stack: 4 = whole attention block in two launches per layer (QKV GEMV, attention + o_proj + "
+                    help="with --stack: 5 = one resident launch for all layers (same work as 2); 4 = whole attention block in two launches per layer (QKV GEMV, attention + o_proj + "
                          "residual in one); 3 = the block in three launches (QKV GEMV, attention, o_proj + residual); "
                          "2 = norm/rope/append fused into the attention launch (default), "
                          "1 = separate kernel before attention (the reference's sequence)")

@@ -82,12 +82,15 @@ def _check_remarks(out, verbose):
         print(out)
 
 
-def build_hip_library(verbose=False, defines=(), output=None):
+def build_hip_library(verbose=False, defines=(), output=None, only=()):
     """`defines`: extra NAME=VALUE macros (the kernels' build-time switches, e.g. LLMI_PV_VALU=1);
-    `output`: where to write a variant build instead of the in-tree library."""
+    `output`: where to write a variant build instead of the in-tree library; `only`: the sources the defines
+    matter to (the others are taken from the in-tree build's objects, which must exist)."""
     tag = "hip" if not (defines or output) else "variant_" + re.sub(r"[^A-Za-z0-9_.-]", "_", os.path.basename(output or "x"))
-    objects, out = _compile_objects([os.path.join(CSRC, s) for s in HIP_SOURCES], list(defines), tag)
+    sources = [s for s in HIP_SOURCES if not only or s in only]
+    objects, out = _compile_objects([os.path.join(CSRC, s) for s in sources], list(defines), tag)
     _check_remarks(out, verbose)
+    objects += [os.path.join(HERE, "build", "hip", s + ".o") for s in HIP_SOURCES if s not in sources]
     return _link_shared(objects, output or LIB_PATH)
 
 
@@ -128,11 +131,13 @@ if __name__ == "__main__":
     ap.add_argument("--define", action="append", default=[], metavar="NAME=VALUE",
                     help="build-time switch of the kernels (LLMI_PV_VALU=1, LLMI_STAGES=3, ...); needs --output")
     ap.add_argument("--output", default=None, help="write a variant of libllmi_hip.so here (load it with LLMI_HIP_LIBRARY)")
+    ap.add_argument("--only", action="append", default=[], metavar="SOURCE",
+                    help="recompile only this source (e.g. mha_stack.hip) for the variant; the rest comes from the in-tree build")
     cli = ap.parse_args()
     if cli.define or cli.output:
         if not cli.output:
             ap.error("--define needs --output: the in-tree library is always the default build")
-        print("built", build_hip_library(verbose=True, defines=cli.define, output=os.path.abspath(cli.output)))
+        print("built", build_hip_library(verbose=True, defines=cli.define, output=os.path.abspath(cli.output), only=cli.only))
         sys.exit(0)
     for p in build_all(verbose=True):
         print("built", p)

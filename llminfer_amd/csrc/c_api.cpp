@@ -449,7 +449,7 @@ static int plan_stack(const llmi_mha_stack_args* args, llmi_mha_plan* plan, bool
     const llmi_mha_args& m = ap.mha;
     if (m.pos_device) return LLMI_OK;
     if (plan->path != LLMI_PATH_SPLIT_FUSED || plan->num_splits < 2 || plan->num_splits > 64) return LLMI_OK;
-    if (plan->group_pad > 4 || plan->waves_per_group != 4) return LLMI_OK;
+    if (plan->group_pad > 4 || plan->waves_per_group != 4 || m.head_num > 64) return LLMI_OK;  // (one lane of the polling wavefront per head)
     if (m.workspace_bytes < plan->workspace_needed + stack_workspace_extra(m.head_num)) return LLMI_OK;
     // every workgroup must be resident at once: workgroups wait for each other
     const int cus = compute_units();

@@ -38,6 +38,40 @@ namespace {
 #define LLMI_STACK_PREFETCH_LATE 0
 #endif
 
+#ifndef LLMI_STACK_SPREAD_MERGE
+#define LLMI_STACK_SPREAD_MERGE 1  // the heads of a KV head are merged by different workgroups (see `spread` below)
+#endif
+#ifndef LLMI_STACK_TIMING_NO_WAIT
+// 1: timing-only build that does not wait for the previous layer's tags (wrong whenever a layer's inputs depend on the
+// layer before): what the order between layers costs. Never the library's build.
+#define LLMI_STACK_TIMING_NO_WAIT 0
+#endif
+
+#ifndef LLMI_STACK_STAMPS
+// 1: diagnostic build that writes the 100 MHz clock at the phases of four layers (LLMI_STACK_STAMP_LAYER ..+3) into the
+// caller's workspace, 4 MiB in (the workspace must be at least 4 MiB + 64 KiB + 16 * grid bytes): per layer and
+// workgroup 16 words -- 0 tags seen, 1 operands landed, 2 tiles done, 3 partial results handed over, 4 records in,
+// 5 partial rows read back, 6 output acknowledged and tag published (4-6: head 0 of a merging workgroup), 8..11 tiles
+// done per wavefront. Never the library's build.
+#define LLMI_STACK_STAMPS 0
+#endif
+#ifndef LLMI_STACK_STAMP_LAYER
+#define LLMI_STACK_STAMP_LAYER 16
+#endif
+#if LLMI_STACK_STAMPS
+#define LLMI_STAMP(slot, cond)                                                                                          \
+    do {                                                                                                                 \
+        const int stamp_l_ = layer - LLMI_STACK_STAMP_LAYER;                                                             \
+        if (stamp_l_ >= 0 && stamp_l_ < 4 && lane == 0 && (cond)) {                                                      \
+            const int stamp_wg_ = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;                                    \
+            const int stamp_i_ = ((stamp_l_ * (int)(gridDim.x * gridDim.y) + stamp_wg_) * 16 + (slot)) & ((1 << 18) - 1); \
+            reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(a.ws) + (4u << 20))[stamp_i_] = (uint32_t)wall_clock64();   \
+        }                                                                                                                \
+    } while (0)
+#else
+#define LLMI_STAMP(slot, cond) do {} while (0)
+#endif
+
 // Copies of a head's done tag, each in a 256-byte line of its own: a workgroup polls copy
 // (its index in the grid) % kDoneCopies, so that a line is polled by a few workgroups instead of all of them.
 #ifndef LLMI_STACK_DONE_COPIES
@@ -65,8 +99,13 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
     const int ntiles = run + (split < longer ? 1 : 0);
     const int begin = (split * run + min(split, longer)) * kTile;
     const int nrows = min(ntiles * kTile, cached_len - begin);
-    const bool merging = split == S - 1;             // this workgroup merges its KV head's splits
-    const bool holds_new_row = merging && wave == 0;  // ... and this wavefront takes the new token
+    // Who merges a query head's splits (log-sum-exp): with at least as many splits as heads in the group, head h's are
+    // merged by wavefront 0 of the workgroup of split S-1-h, so that the heads' read-backs run on different compute
+    // units at the same time; else the workgroup of the last split merges every head, a wavefront each.
+    const bool spread = LLMI_STACK_SPREAD_MERGE && S >= a.group;
+    const int merge_head = spread ? (S - 1 - split < a.group ? S - 1 - split : -1) : -1;
+    const bool merges_any = spread ? merge_head >= 0 : split == S - 1;
+    const bool holds_new_row = split == S - 1 && wave == 0;  // this wavefront takes the new token
 
     const int64_t split_off = (int64_t)kvh * a.head_stride + (int64_t)begin * a.row_stride;
     const uint32_t rs = (uint32_t)a.row_stride * 2u;
@@ -92,7 +131,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
     constexpr int kMergeBytes = NW * G * kHeadDim * (int)sizeof(float);
     constexpr int kTailFloats = 2 * NW * G + 2 * G + G * 64 + 4;
     constexpr int kSmemBytes = kRingBytes + kStagingBytes + kMergeBytes + kTailFloats * 4;
-    static_assert(kSmemBytes <= 80 * 1024, "two workgroups' worth of LDS per CU keeps the VGPR-form matrix instructions");
+    static_assert(NW > 4 || kSmemBytes <= 80 * 1024, "two workgroups' worth of LDS per CU keeps the VGPR-form matrix instructions");
+    static_assert(kSmemBytes <= 160 * 1024, "LDS of one compute unit");
     __shared__ __attribute__((aligned(1024))) char smem[kSmemBytes];
     char* my_ring = smem + wave * kWaveRingBytes;
     const uint32_t my_ring_lds = (uint32_t)(uintptr_t)my_ring;
@@ -154,7 +194,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
     // Where this split's partial results and records go (the same rows in every layer: a layer's are consumed
     // before the next layer's are written, and a record names its layer by its tag).
     const int my_xs = package_side<BYSIDE>();
-    const int store_xs = my_xs ^ (int)(BYSIDE && !merging && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
+    const int store_xs = my_xs ^ (int)(BYSIDE && !merges_any && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * S + 15) & ~(int64_t)15) : (int64_t)a.n_q * S;
     const int part_bytes = (int)(part_rows * kHeadDim * (int64_t)sizeof(float));
     const __amdgpu_buffer_rsrc_t part_rsrc = __builtin_amdgcn_make_buffer_rsrc(a.ws, 0, part_bytes, 0x00020000);
@@ -165,6 +205,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
     const WsHead u_wh = ws_head<BYSIDE>(a, u_hq);
     const uint32_t u_po = (uint32_t)(((int64_t)ws_row<4>(u_wh, split, store_xs) * kHeadDim + u_c4 * 4) * (int64_t)sizeof(float));
     const int64_t u_rec = (int64_t)ws_row<9>(u_wh, split, store_xs) * 2;
+    const bool u_own = spread ? merge_head == u_h : split == S - 1;  // this workgroup merges the unit's head itself
 
     // The done tags: copy c of head h at done[c * words_per_copy + h].
     const int words_per_copy = ((a.n_q + kDoneLineWords - 1) / kDoneLineWords) * kDoneLineWords;
@@ -177,14 +218,15 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
     for (int layer = 0; layer < sa.layers; ++layer) {
         const uint32_t tag = 0x80000000u | ((a.tag + (uint32_t)layer) & 0x7fffffffu);
         // ---- (1) the previous layer is done: every query head carries its tag ----
-        if (layer > 0 && wave == 0 && !poisoned) {  // (after a give-up nothing is waited for any more: the rest is NaN anyway)
+        if (!LLMI_STACK_TIMING_NO_WAIT && layer > 0 && wave == 0 && !poisoned) {  // (after a give-up nothing is waited for any more: the rest is NaN anyway)
             const uint32_t want = 0x80000000u | ((a.tag + (uint32_t)layer - 1u) & 0x7fffffffu);
             bool seen = false;
-            for (int spin = 0; spin < a.max_polls && !seen; ++spin) {
-                const uint32_t d0 = __hip_atomic_load(my_done + min(lane, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const uint32_t d1 = __hip_atomic_load(my_done + min(lane + 64, a.n_q - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                seen = __all(d0 == want && d1 == want);
-            }
+            // (one poll at a time, back to back: two, four or eight polls in flight a fraction of a round trip apart see a
+            // tag sooner on paper, and measured 0.06, 0.17 and 0.34 us per layer SLOWER -- polls are traffic on the lines
+            // the tags have to reach)
+            const uint32_t* tag_ptr = my_done + min(lane, a.n_q - 1);
+            for (int spin = 0; spin < a.max_polls && !seen; ++spin)
+                seen = __all(__hip_atomic_load(tag_ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want);
             if (lane == 0) {
                 *s_flag = seen ? 1 : 0;
                 if (!seen) atomicAdd(&g_poll_timeouts, 1u);
@@ -192,7 +234,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
         }
         // (also: every wavefront is through with the previous layer's merge area and staging slots)
         __syncthreads();
-        if (layer > 0 && *s_flag == 0) poisoned = true;
+        if (!LLMI_STACK_TIMING_NO_WAIT && layer > 0 && *s_flag == 0) poisoned = true;
+        LLMI_STAMP(0, wave == 0);
 
         // ---- (2) this layer's small operands, by DMA into the staging slots ----
         const uint16_t* q_l = a.q + (int64_t)layer * sa.q_stride;
@@ -221,6 +264,8 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
         // (loads complete in order: the tiles requested earlier are in their slots as well)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         u32x4 qb[4];
+        u32x4 new_k[4], new_v;  // the new token's K row (operand layout) and V row, in the wavefront that holds it
+        LLMI_STAMP(1, wave == 0);
         float m_run = -INFINITY, l_run = 0.0f;
         f32x4 o[8];
 #pragma unroll
@@ -248,13 +293,9 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) kf[j] = sh4[64 + j * 4 + kg];
                 const u32x4 vf = sh4[64 + 16 + n16];
-                const int64_t row_off = (int64_t)layer * sa.cache_stride + (int64_t)(seq_len - 1) * a.row_stride + kvh * a.slot_head_stride;
-                if (n16 == 0) {
-                    uint16_t* kd = const_cast<uint16_t*>(a.k) + row_off;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = kf[j];
-                }
-                if (kg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + row_off + n16 * 8) = vf;
+                for (int j = 0; j < 4; ++j) new_k[j] = kf[j];
+                new_v = vf;  // (filed in the cache behind the tiles: the stores' acknowledgement must not sit in front of a tile's wait)
                 float dot = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -332,6 +373,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
             for (int j = 0; j < 8; ++j) o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pb, vb4[j], o[j], 0, 0, 0);
         }
 
+        if (holds_new_row) {
+            const int64_t row_off = (int64_t)layer * sa.cache_stride + (int64_t)(seq_len - 1) * a.row_stride + kvh * a.slot_head_stride;
+            if (n16 == 0) {
+                uint16_t* kd = const_cast<uint16_t*>(a.k) + row_off;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(kd + (j * 4 + kg) * 8) = new_k[j];
+            }
+            if (kg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + row_off + n16 * 8) = new_v;
+        }
+        LLMI_STAMP(2, wave == 0);
+        LLMI_STAMP(8 + wave, true);
         // ---- (4) fold the workgroup's wavefronts, hand the split's partial results over ----
         l_run = rows_sum(l_run);
         if (kg == 0) {
@@ -372,7 +424,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
             }
             if (poisoned) lsum = __builtin_nanf("");
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), part_rsrc, u_po, 0, kCacheDevice);
-            if (!merging) {
+            if (!u_own) {
                 // the head's record goes out as soon as this wavefront's stores are acknowledged (the 32 columns of a
                 // head are stored by one half of one wavefront)
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -389,16 +441,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
                 s_fin[2 * u_h + 1] = lsum;
             }
         }
+        LLMI_STAMP(3, wave == 0);
         if (LLMI_STACK_PREFETCH_LATE) {
             while (in_flight < NSTAGE && iss_layer < sa.layers && n_my > 0) issue_next();
         }
-        if (!merging) continue;
+        if (!merges_any) continue;
 
-        // ---- (5) the workgroup of the head's last split merges the splits (log-sum-exp), one wavefront per head ----
+        // ---- (5) the log-sum-exp merge of a head's splits, one wavefront per head ----
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // its own partial stores are acknowledged
         __syncthreads();                                  // ... and its (max, sum) pairs are in LDS
-        if (wave < a.group) {
-            const int h = wave;
+        if (spread ? wave == 0 : wave < a.group) {
+            const int h = spread ? merge_head : wave;
             const int c4 = lane & 31, part = lane >> 5;
             const int hq = kvh * a.group + h;
             const WsHead wh = ws_head<BYSIDE>(a, hq);
@@ -412,7 +465,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
                 ok = true;
                 m_reg = -INFINITY;
                 l_reg = 0.0f;
-                if (lane < S - 1) {
+                if (lane < S && lane != split) {
                     const unsigned long long* rec = rec_near;
                     unsigned long long r0 = __hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     unsigned long long r1 = __hip_atomic_load(rec + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -430,7 +483,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
                     ok = here;
                     m_reg = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
                     l_reg = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
-                } else if (lane == S - 1) {
+                } else if (lane == split) {
                     m_reg = s_fin[2 * h];
                     l_reg = s_fin[2 * h + 1];
                 }
@@ -450,6 +503,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
             }
             const bool arrived = __all(ok);
             if (__builtin_expect(!arrived, 0) && lane == 0) atomicAdd(&g_poll_timeouts, 1u);
+            LLMI_STAMP(4, wave == 0);
 
             const uint32_t row0_bytes = (uint32_t)wh.rbase * (kHeadDim * 4u);
             const uint32_t block_mask = BYSIDE ? ~(uint32_t)(kSideBlockBytes - 1) : 0u;
@@ -477,7 +531,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
             float* w = s_w + h * 64;
             if (lane < S) {
                 w[lane] = f;
-                if (lane < S - 1) {  // consumed: cleared, so that a replay of this launch (same tags) starts clean
+                if (lane != split) {  // consumed: cleared, so that a replay of this launch (same tags) starts clean
                     unsigned long long* rec = a.records + (int64_t)ws_row<9>(wh, lane, home ? 1 : 0) * 2;
                     __hip_atomic_store(rec, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(rec + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -503,6 +557,7 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) sum[e] = halves_sum(sum[e]);
+            LLMI_STAMP(5, wave == 0);
             if (part == 0) {
                 const float inv = (arrived && !poisoned) ? 1.0f / den : __builtin_nanf("");
                 const f32x4 r = sum * inv;
@@ -522,13 +577,17 @@ __global__ __launch_bounds__(NW * 64, 2) void mha_stack_kernel(StackArgs sa) {
                 if (lane < kDoneCopies)
                     __hip_atomic_store(sa.done + (size_t)lane * words_per_copy + hq, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+            LLMI_STAMP(6, wave == 0);
         }
     }
 }
 
 template <int G>
 bool launch_stack_g(const StackArgs& sa, int n_kv, hipStream_t stream) {
-    constexpr int NW = 4, NSTAGE = 2;
+#ifndef LLMI_STACK_WAVES
+#define LLMI_STACK_WAVES 4
+#endif
+    constexpr int NW = LLMI_STACK_WAVES, NSTAGE = 8 / NW;  // the rings hold eight tiles per workgroup either way
     const dim3 grid(n_kv, sa.a.num_splits), block(NW * 64);
     if (sa.a.by_side) hipLaunchKernelGGL((mha_stack_kernel<G, NW, NSTAGE, true>), grid, block, 0, stream, sa);
     else hipLaunchKernelGGL((mha_stack_kernel<G, NW, NSTAGE, false>), grid, block, 0, stream, sa);
@@ -538,7 +597,7 @@ bool launch_stack_g(const StackArgs& sa, int n_kv, hipStream_t stream) {
 }  // namespace
 
 bool launch_stack(const StackArgs& sa, int n_kv, int group_pad, int waves, hipStream_t stream) {
-    if (waves != 4) return false;
+    if (waves != 4) return false;  // (the plan's wave count; the kernel's own is LLMI_STACK_WAVES)
     switch (group_pad) {
         case 1: return launch_stack_g<1>(sa, n_kv, stream);
         case 2: return launch_stack_g<2>(sa, n_kv, stream);
