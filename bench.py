@@ -71,13 +71,16 @@ def make_arena(torch, dev, ctx_list, n_q=N_Q):
     return k, v, q, regions
 
 
+KERNEL_SOURCES = ("mha_decode_kernels.h", "mha_device_helpers.h", "mha_decode.hip", "c_api.cpp")
+
+
 def kernel_source_blob():
-    """git's blob ids of the decode kernel's source and of the dispatcher's (what `git rev-parse
-    HEAD:llminfer_amd/csrc/mha_decode.hip` and `...:c_api.cpp` print for committed files), computed from the
-    files themselves and joined by a '+': the kernel and the plan it is launched with decide the traffic."""
+    """git's blob ids of the decode kernel's sources and of the dispatcher's (what `git rev-parse
+    HEAD:llminfer_amd/csrc/<file>` prints for committed files), computed from the files themselves and joined
+    by a '+': the kernel and the plan it is launched with decide the traffic."""
     import hashlib
     ids = []
-    for name in ("mha_decode.hip", "c_api.cpp"):
+    for name in KERNEL_SOURCES:
         data = open(os.path.join(ROOT, "llminfer_amd", "csrc", name), "rb").read()
         ids.append(hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest())
     return "+".join(ids)
@@ -405,14 +408,14 @@ class Sweep:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1)
 
-    def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None, steps=SLICES):
-        """Best of `reps` batches of graph replays (a graph of `steps` steps), us per call."""
+    def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None, steps=SLICES, stat="best"):
+        """Best (or, stat="all", every one) of `reps` batches of graph replays (a graph of `steps` steps), us per call."""
         g = self.capture(enqueue_fn, steps)
         scale = max(1, steps // SLICES)
         self.time_replays([(g, max(1, 8 // scale))])
         n = max(1, (replays or 40) // scale)
-        best = min(self.time_replays([(g, n)]) for _ in range(reps))
-        return best * 1e3 / (n * steps * calls_per_step)
+        samples = [self.time_replays([(g, n)]) * 1e3 / (n * steps * calls_per_step) for _ in range(reps)]
+        return samples if stat == "all" else min(samples)
 
 
 # stream-only configurations tried for the floor: (workgroups, waves per workgroup, tiles in flight per wave)
@@ -444,27 +447,33 @@ DISPATCH_CTX = [96, 160, 176, 300, 700, 1024, 1500, 3000, 4097, 5000, 9000, 1234
 
 def dispatch_rows(sw, ctx_list):
     """What the dispatcher picks against forced alternatives, per context length: single pass, and the fused
-    split path at several split counts; same timing method as the per-context figures."""
+    split path at several split counts; same timing method as the per-context figures. Every plan -- the automatic
+    one and each forced one -- is timed equally often (two rounds over all plans, three batches of graph replays
+    each) and judged by the MEDIAN of its six batches."""
     B = sw.B
     rows = []
     for ctx in ctx_list:
         def timed(**over):
-            return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over), steps=n_slices(ctx))
-        timed()  # the first graph timed on a context's slices runs up to a microsecond per call slow: discard one
-        auto = timed()
-        alts = {}
+            return sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n, **over), steps=n_slices(ctx), stat="all")
+        plans = {"auto": {}}
         if ctx <= 1024:
-            alts["single"] = timed(force_path=B.PATH_SINGLE_PASS)
+            plans["single"] = dict(force_path=B.PATH_SINGLE_PASS)
         tiles = (ctx + 15) // 16
         for sp in (4, 8, 16, 32, 64):
             if sp <= tiles:
-                alts["split%d" % sp] = timed(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
-        auto = min(auto, timed())  # (and once more at the end: the automatic plan is one of the forced ones)
-        best = min(alts, key=alts.get)
+                plans["split%d" % sp] = dict(force_path=B.PATH_SPLIT_FUSED, num_splits=sp)
+        timed()  # the first graph timed on a context's slices runs up to a microsecond per call slow: discard one
+        samples = {name: [] for name in plans}
+        for _ in range(2):
+            for name, over in plans.items():
+                samples[name] += timed(**over)
+        med = {name: sorted(v)[len(v) // 2] for name, v in samples.items()}
+        auto = med.pop("auto")
+        best = min(med, key=med.get)
         p = sw.plan(ctx)
         rows.append({"ctx": ctx, "auto_us": round(auto, 2), "auto_plan": "path%d S=%d W=%d" % (p.path, p.num_splits, p.waves_per_group),
-                     "best_forced": best, "best_forced_us": round(alts[best], 2), "auto_over_best": round(auto / alts[best], 3),
-                     "forced_us": {k2: round(v2, 2) for k2, v2 in alts.items()}})
+                     "best_forced": best, "best_forced_us": round(med[best], 2), "auto_over_best": round(auto / med[best], 3),
+                     "forced_us": {k2: round(v2, 2) for k2, v2 in med.items()}})
     return rows
 
 
@@ -692,6 +701,9 @@ def main():
                      "ms_per_step_median": round(median_ms, 6), "value_median": round(step_bytes / (median_ms * 1e-3) / 1e9, 1),
                      "ms_per_step_p10": round(batch_ms[len(batch_ms) // 10], 6), "ms_per_step_p90": round(batch_ms[len(batch_ms) * 9 // 10], 6)},
         "us_per_layer_mean": round(avg_launch_us, 3),
+        "per_ctx_stat": "per_ctx, position_major, stream_floor and cfg5 figures: best of 3 (floor: 2) batches of graph replays of one "
+                        "length alone; dispatch_check: median of 6 batches per plan; value, ms_per_step and roofline: the timed "
+                        "region itself, nothing picked",
         "per_ctx": per_ctx,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
@@ -706,6 +718,7 @@ def main():
         for row, f in zip(per_ctx, floor):
             row["stream_floor_us"] = f["us"]
             row["stream_floor_frac_peak"] = f["frac_peak"]
+            row["floor_ratio"] = round(f["us"] / row["us_per_layer"], 3)  # stream-only floor / decode kernel: 1 = at the floor
         result["stream_floor"] = floor
         del sw
         torch.cuda.empty_cache()
@@ -715,12 +728,14 @@ def main():
             result["position_major"] = per_ctx_rows(sw_pm, ctx_list, 40)
             for row, f in zip(result["position_major"], stream_floor(sw_pm, ctx_list)):  # the same pieces, read and thrown away
                 row["stream_floor_us"] = f["us"]
+                row["floor_ratio"] = round(f["us"] / row["us_per_layer"], 3)
             del sw_pm
             torch.cuda.empty_cache()
             # the dispatch against forced plans at lengths either side of the threshold, powers of two and not
             sw_d = Sweep(DISPATCH_CTX, n_q, 1)
             rows = dispatch_rows(sw_d, DISPATCH_CTX)
-            result["dispatch_check"] = {"worst_auto_over_best": max(r["auto_over_best"] for r in rows),
+            result["dispatch_check"] = {"stat": "median of 6 batches per plan, automatic and forced plans timed equally often",
+                                        "worst_auto_over_best": max(r["auto_over_best"] for r in rows),
                                         "rows": [{k2: r[k2] for k2 in ("ctx", "auto_us", "auto_plan", "best_forced", "best_forced_us", "auto_over_best")}
                                                  for r in rows]}
             del sw_d
@@ -730,16 +745,21 @@ def main():
             r5 = per_ctx_rows(sw5, [131072], 10)[0]
             f5 = stream_floor(sw5, [131072], FLOOR_CONFIGS[:4])[0]
             result["cfg5"] = dict(r5, workload="64 Q / 8 KV heads, ctx 131072, head-major, graph replays over %d KV slices" % SLICES,
-                                  stream_floor_us=f5["us"])
+                                  stream_floor_us=f5["us"], floor_ratio=round(f5["us"] / r5["us_per_layer"], 3))
             del sw5
             torch.cuda.empty_cache()
             # BASELINE config 4: 36 layers at ctx 4096 + 1 new token, fused QK-Norm + RoPE + append, one HIP graph per token
-            ns = argparse.Namespace(stack=36, heads=32, layout=1, stack_mode=2, stack_follow_pos=False, steps=200, warmup=20)
+            ns = argparse.Namespace(stack=36, heads=32, layout=1, stack_mode=5, stack_follow_pos=False, steps=200, warmup=20)
             r4 = stack_result(ns, 4096)
-            if r4 is not None:
+            ns.stack_mode = 2
+            r4b = stack_result(ns, 4096)
+            if r4 is not None and r4b is not None:
                 result["cfg4_stack"] = {"us_per_token": r4["value"], "us_per_layer": r4["us_per_layer"],
                                         "frac_peak": r4["roofline"]["frac"], "GBps": r4["roofline"]["achieved"],
-                                        "workload": r4["config"]["workload"]}
+                                        "workload": r4["config"]["workload"],
+                                        "one_launch_per_layer": {"us_per_token": r4b["value"], "us_per_layer": r4b["us_per_layer"],
+                                                                 "frac_peak": r4b["roofline"]["frac"],
+                                                                 "workload": r4b["config"]["workload"]}}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(ctx_list, n_q=n_q)
     print(json.dumps(result))
