@@ -107,6 +107,16 @@ int poll_limit() { return g_poll_limit.load(std::memory_order_relaxed); }
 static std::atomic<int> g_test_far_home{0};
 int test_far_home() { return g_test_far_home.load(std::memory_order_relaxed); }
 
+// With 32 splits and more (16 for groups of eight query heads) the merge of a KV head's query heads is spread over as
+// many workgroups; with fewer, the workgroup of the last split merges them all. Measured, 32 Q / 8 KV heads, spread
+// against not: 16 splits 5.08 : 4.98 us at 1024 positions, 5.87 : 5.77 at 2048; 8 splits 4.51 : 4.41 at 256; 32 splits
+// 5.03 : 5.14 at 1024, 5.71 : 5.80 at 2048, 6.86 : 7.08 at 4096, 7.88 : 8.10 at 6000; 64 Q heads, 16 splits 5.55 : 5.68 at
+// 1024, 7.63 : 7.81 at 4096, 32 splits at 32768 24.4 : 25.3. LLMI_HIP_SPREAD_MIN_SPLITS moves the boundary.
+int spread_merge_min_splits(int group_pad) {
+    static const int v = env_int("LLMI_HIP_SPREAD_MIN_SPLITS", 1, 1 << 20, 0);
+    return v ? v : group_pad >= 8 ? 16 : 32;
+}
+
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
 
 static int validate_mha(const llmi_mha_args* a) {
@@ -196,16 +206,15 @@ static int make_plan(const llmi_mha_args* a, llmi_mha_plan* p, int wave_cap = kM
             if (half < 2) half = 2;
             int quarter = half / 2;
             if (quarter < 2) quarter = 2;
-            // With 8 waves per workgroup (one LDS stage per wave) a split wants two tiles per wave before
-            // one workgroup per CU pays (64 query / 8 KV heads, 16 against 32 splits: 5.55 : 6.42 us at 512
-            // positions, 6.75 : 7.31 at 2048, 8.08 : 8.63 at 4096, level at 8192, 27.2 : 24.9 at 32768).
-            // With 4 waves the smaller grid keeps the lead while its wavefronts have up to three tiles each (two in the
-            // position-major layout): half as many partials to read back outweighs the shorter runs. 32 query / 8 KV
-            // heads, workspace laid out by package side, 16 against 32 splits: 5.23 : 5.42 us at 1024 positions,
-            // 5.96 : 6.13 at 2048, 6.70 : 6.79 at 3000, 7.31 : 7.38 at 4096, 8.01 : 7.96 at 5000, 10.16 : 9.65 at 8192;
-            // position-major 6.12 : 6.18 at 2048, 7.16 : 7.05 at 3000, 7.85 : 7.59 at 4096.
-            const int per_wave = a->kv_layout == LLMI_KV_LAYOUT_HEAD_MAJOR ? 3 : 2;
-            const int full = waves == 8 ? target * 16 : half * waves * per_wave + 1;
+            // One workgroup per CU pays as soon as half as many splits would hold more than four tiles each (more than
+            // one per wavefront at four wavefronts). Measured with the merge of a KV head's query heads spread over
+            // several workgroups (which needs 32 splits to pay at groups of four, see spread_merge_min_splits), 32 Q / 8 KV
+            // heads, head-major, 16 against 32 splits: 4.98 : 5.03 us at 1024 positions, 5.43 : 5.16 at 1200, 5.51 : 5.44 at
+            // 1500, 5.69 : 5.60 at 1800, 5.77 : 5.71 at 2048, 6.49 : 6.40 at 3000, 7.16 : 6.86 at 4096; position-major 4.96 : 5.07
+            // at 1024, 5.54 : 5.43 at 1500, 5.84 : 5.69 at 2048, 6.71 : 6.46 at 3000, 7.41 : 6.93 at 4096; 64 Q / 8 KV heads
+            // (8 wavefronts) 5.09 : 5.22 at 512, 5.55 : 5.51 at 1024, 6.35 : 6.13 at 2048, 7.63 : 7.43 at 4096, 10.45 : 9.67 at
+            // 8192, 16.07 : 14.72 at 16384.
+            const int full = half * 4 + 1;
             want = tiles >= full ? target : tiles >= half ? half : quarter;
             if (want > tiles) want = tiles;
             if (cap < 2) return LLMI_ERR_WORKSPACE;

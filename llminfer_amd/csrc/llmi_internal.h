@@ -65,6 +65,8 @@ inline size_t side_pad(const void* workspace) { return (size_t)(-reinterpret_cas
 constexpr bool by_side_variant(int group_pad, int waves) { return group_pad <= 8 && waves == (group_pad == 8 ? 8 : 4); }
 // Waits of the fused combine that gave up since the library was loaded (device counter of the current device).
 int read_poll_timeouts(unsigned long long* count);
+// Fewest splits at which the fused combine hands the heads of a KV head to different workgroups.
+int spread_merge_min_splits(int group_pad);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.
 int poll_limit();
 // Testing aid (llmi_hip_set_test_far_home): 1 = every split but the merging one, 2 = every second split stores into

@@ -182,6 +182,7 @@ static int fill_kernel_args(const llmi_mha_args& args, const llmi_mha_plan& plan
         ka.head_stride = (int64_t)args.max_seq_len * args.head_dim;
     }
     ka.seq_len = args.pos + 1;
+    ka.spread_merge = plan.num_splits >= spread_merge_min_splits(plan.group_pad);
     ka.max_polls = poll_limit();
     ka.stagger = args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR;
     ka.group = args.kv_mul;

@@ -50,6 +50,7 @@ struct KernelArgs {
     // partial outputs / records; XCDs 4-7 use the other one.
     bool by_side;
     unsigned long long ppar[2], rpar[2];
+    bool spread_merge;  // fused combine: the heads of a KV head are merged by different workgroups (the host's choice, by split count)
     int32_t far_home;  // testing aid: 1 = every split but the merging one, 2 = every second one uses the other side's home
 };
 

@@ -72,6 +72,7 @@ constexpr int kWavesPerEu = (G >= 16 && NW != 2) ? 1 : LLMI_MIN_WAVES_PER_EU;
 
 template <int G, int NW, int NSTAGE, bool APPEND, bool DYN, bool STAGGER, bool OPROJ, bool BYSIDE>
 __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState& proj) {
+    constexpr bool kSpreadMerge = LLMI_SPREAD_MERGE && !OPROJ && G <= NW;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: loop control stays on the SALU
     const int n16 = lane & 15;  // MFMA column / DPP-row lane
@@ -372,8 +373,15 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     // path of whoever waits for this split (the empty asm statements keep the compiler from moving the work there).
     const bool fused = a.records != nullptr && n_active > 1;
     const int my_xs = package_side<BYSIDE>();  // wave-uniform: the side of the package this workgroup runs on
-    // (testing aid: pretend this split ran on the other side; never the merging one, whose own rows it reads itself)
-    const int store_xs = my_xs ^ (int)(BYSIDE && split != n_active - 1 && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
+    // Who merges a query head's splits (log-sum-exp): where one wavefront merges a head (G <= NW) and there are at
+    // least as many splits as heads in the group, head h's splits are merged by wavefront 0 of the workgroup of split
+    // SA-1-h, so that the heads' read-backs (16 KiB each at 32 splits) run on different compute units at the same
+    // time instead of queueing at one; otherwise the workgroup of the last split merges every head.
+    const bool spread = kSpreadMerge && a.spread_merge && n_active >= a.group;
+    const int merge_head = spread && n_active - 1 - split < a.group ? n_active - 1 - split : -1;
+    const bool merges_any = spread ? merge_head >= 0 : split == n_active - 1;
+    // (testing aid: pretend this split ran on the other side; never a merging one, whose own rows it reads itself)
+    const int store_xs = my_xs ^ (int)(BYSIDE && !merges_any && (a.far_home == 1 || (a.far_home == 2 && (split & 1))));
     const int n_units = a.group * (kHeadDim / 4);
     const int64_t part_rows = BYSIDE ? 2 * (((int64_t)a.n_q * a.num_splits + 15) & ~(int64_t)15) : (int64_t)a.n_q * a.num_splits;
     int part_bytes = (int)(part_rows * kHeadDim * (int64_t)sizeof(float));
@@ -554,7 +562,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 // anyone flushing or invalidating a cache.
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc), part_rsrc,
                                                        (uint32_t)(po * (int64_t)sizeof(float)), 0, 16);
-                if (split != n_active - 1) {
+                if (spread ? h != merge_head : split != n_active - 1) {
                     // Publish the head's record as soon as this wavefront's stores are acknowledged:
                     // the 32 columns of a head are stored by one half of one wavefront, so no
                     // workgroup barrier is needed.
@@ -567,7 +575,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                         __hip_atomic_store(rec, tag | (m_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         __hip_atomic_store(rec + 1, tag | (l_bits << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
-                } else if (c4 == 0) {  // the combiner keeps its own pair in LDS
+                } else if (c4 == 0) {  // the workgroup that merges this head keeps its own pair in LDS
                     s_fin[2 * h] = mx;
                     s_fin[2 * h + 1] = lsum;
                 }
@@ -596,7 +604,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     // graph replay of this very call (same epoch) starts clean.
     const int S = a.num_splits;  // layout stride of partials and records
     const int SA = n_active;     // splits that hold positions
-    if (split != SA - 1) return;  // (its records went out above)
+    if (!merges_any) return;  // (its records went out above)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the combiner's own partial stores are acknowledged
     __syncthreads();                                  // ... and its (max, sum) pairs are in LDS
 
@@ -633,7 +641,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 const int sp = lane + 64 * j;
                 m_reg[j] = -INFINITY;
                 l_reg[j] = 0.0f;
-                if (sp < SA - 1) {
+                if (sp < SA && sp != split) {
                     const unsigned long long* rec = rec_near[j];
                     unsigned long long r0 = __hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     unsigned long long r1 = __hip_atomic_load(rec + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -651,7 +659,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                     ok = ok && here;
                     m_reg[j] = __builtin_bit_cast(float, (uint32_t)(r0 >> 32));
                     l_reg[j] = __builtin_bit_cast(float, (uint32_t)(r1 >> 32));
-                } else if (sp == SA - 1) {
+                } else if (sp == split) {
                     m_reg[j] = s_fin[2 * h];
                     l_reg[j] = s_fin[2 * h + 1];
                 }
@@ -695,7 +703,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
                 const float f = (m_reg[j] == -INFINITY) ? 0.0f : fast_exp2(m_reg[j] - mx);
                 s_w[h * kMaxSplits + sp] = f;
                 den += l_reg[j] * f;
-                if (sp < SA - 1) {
+                if (sp != split) {
                     unsigned long long* rec = a.records + (int64_t)ws_row<9>(wh, sp, home[j] ? 1 : 0) * 2;
                     __hip_atomic_store(rec, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(rec + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -726,8 +734,8 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
         // with one lane swap. The partials of the other workgroups were acknowledged before
         // their records were written; they are read with device-coherent 16-byte loads, a
         // lane's loads all in flight at once.
-        if (wave >= a.group) return;
-        const int h = wave;
+        if (spread ? wave != 0 : wave >= a.group) return;
+        const int h = spread ? merge_head : wave;
         const int c4 = lane & 31;
         const int part = lane >> 5;
         const int hq = kvh * a.group + h;

@@ -49,6 +49,11 @@ constexpr int kCacheDevice = 16;
 // attention output; the others are requested after the wait.
 #define LLMI_OPROJ_PREFETCH_ROWS 3
 #endif
+#ifndef LLMI_SPREAD_MERGE
+// 1: the heads of a KV head are merged by different workgroups of the split path (see `spread` in mha_decode_body);
+// 0: by the workgroup of the last split, a wavefront each. Kept for the side-by-side measurement.
+#define LLMI_SPREAD_MERGE 1
+#endif
 #ifndef LLMI_PV_VALU
 // 1: the probability x value product runs on the vector ALU (fp32 multiply-adds with the
 // probabilities broadcast by DPP, the structure of the reference's inner loop,

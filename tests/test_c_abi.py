@@ -144,14 +144,23 @@ def test_plan_long_context_splits_without_empty_splits(ctx):
     assert p.group_pad == 4 and p.waves_per_group in (1, 2, 4, 8)
 
 
+def test_plan_split_count_by_length():
+    """32 query / 8 KV heads: 8 splits while 16 would leave some without a tile, 16 until they would hold more than four
+    tiles each (1024 positions), then one workgroup per CU, in both layouts."""
+    for layout in (0, 1):
+        for ctx, splits in ((177, 8), (240, 8), (241, 16), (700, 16), (1024, 16), (1025, 32), (1041, 32), (1500, 32), (3000, 32), (4096, 32), (32768, 32)):
+            rc, p = plan(good_args(pos=ctx - 1, max_seq_len=32768, kv_layout=layout))
+            assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and p.num_splits == splits, (layout, ctx, p.num_splits)
+
+
 def test_plan_groups_of_eight_query_heads():
-    """64 query / 8 KV heads: 8 waves per workgroup, a single pass up to 240 positions (15 tiles), then one
-    workgroup per CU and KV head pair (16 splits) until a split's run is long enough for 32."""
+    """64 query / 8 KV heads: 8 waves per workgroup, a single pass up to 240 positions (15 tiles), then 16 splits
+    until they would hold more than four tiles each (1024 positions), then one workgroup per CU (32 splits)."""
     eight = dict(kv_mul=8, head_num=64, max_seq_len=32768)
     for pos in (0, 127, 208, 239):
         rc, p = plan(good_args(pos=pos, **eight))
         assert rc == 0 and p.path == B.PATH_SINGLE_PASS and p.num_splits == 1 and p.group_pad == 8
-    for ctx, splits in ((241, 16), (256, 16), (1024, 16), (4096, 16), (8192, 32), (32768, 32)):
+    for ctx, splits in ((241, 16), (256, 16), (1024, 16), (1025, 32), (1041, 32), (4096, 32), (8192, 32), (32768, 32)):
         rc, p = plan(good_args(pos=ctx - 1, **eight))
         assert rc == 0 and p.path == B.PATH_SPLIT_FUSED and p.waves_per_group == 8
         assert p.num_splits == splits and p.rows_per_split == -(-((ctx + 15) // 16) // splits) * 16
