@@ -505,6 +505,46 @@ def run_calibrate_hbm(args):
     return 0
 
 
+STREAM_MODES = ["registers, linear", "LDS-DMA, linear", "LDS-DMA, K swizzled (the decode kernel's requests)",
+                "LDS-DMA, K swizzled, pause after every tile"]
+
+
+def run_stream_variants(args, ctx_list):
+    """The decode kernel's K/V stream without its arithmetic, one feature at a time (llmi_hip_probe_stream_tiles), on the decode
+    kernel's own grid of 32 splits x 8 KV heads, next to the decode kernel itself: which feature of the request pattern costs
+    bandwidth, in both cache layouts. Same graph-replay timing and rotating KV slices as the headline figures."""
+    import torch
+    from llminfer_amd import _binding as B
+    from llminfer_amd import ops
+    n_q = args.heads
+    waves, inflight = (8, 1) if n_q // N_KV >= 8 else (4, 2)
+    probe = B.lib().llmi_hip_probe_stream_tiles
+    rows = []
+    for layout in (1, 0):
+        sw = Sweep(ctx_list, n_q, layout)
+        for ctx in ctx_list:
+            decode_us = sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n), reps=3, replays=40, steps=n_slices(ctx))
+            row = {"ctx": ctx, "layout": "head-major" if layout == 1 else "position-major", "splits": 32, "waves": waves,
+                   "tiles_in_flight": inflight, "decode_us": round(decode_us, 2), "variants": []}
+            for mode, pause, stagger in ((0, 0, 0), (1, 0, 0), (2, 0, 0), (3, 4, 0), (3, 8, 0), (3, 16, 0)) + (((2, 0, 1),) if layout == 0 else ()):
+                def enq(first, n):
+                    for st in range(first, first + n):
+                        off = sw.regions[(ctx, st % n_slices(ctx))] * 2
+                        B.check(probe(sw.k.data_ptr() + off, sw.v.data_ptr() + off, ctx, N_KV, layout, 32, waves, inflight, mode, pause,
+                                      stagger, sw.sink.data_ptr(), sw.stream.cuda_stream), "llmi_hip_probe_stream_tiles")
+                us = sw.us_per_call(enq, reps=3, replays=40, steps=n_slices(ctx))
+                row["variants"].append({"mode": STREAM_MODES[mode] + (" (%d x 64 clocks)" % pause if mode == 3 else "") +
+                                                (", staggered walk" if stagger else ""),
+                                        "us": round(us, 2), "TBps": round(2 * ctx * KV_DIM * 2 / us / 1e6, 3)})
+            rows.append(row)
+        del sw
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": "K/V stream variants next to the decode kernel, us per launch (graph replays, best of 3 batches)", "n_gpus": 1,
+                      "config": {"workload": "%d Q / 8 KV heads; K and V rows of one call read once and thrown away by a kernel with the decode "
+                                             "kernel's grid and tile deal" % n_q}, "rows": rows}))
+    return 0
+
+
 def run_placement(args):
     """Where the workgroups of a 128 / 256 / 512-workgroup launch with a decode workgroup's footprint land."""
     import collections
@@ -569,6 +609,9 @@ def main():
                     help="time the automatic plan against forced single-pass / split plans at every --ctx")
     ap.add_argument("--stream-floor", action="store_true",
                     help="time a kernel that only reads the same K/V bytes, next to the decode kernel, at every --ctx")
+    ap.add_argument("--stream-variants", action="store_true",
+                    help="time the decode kernel's K/V stream without its arithmetic, one feature of the request pattern at a time, "
+                         "in both cache layouts, at every --ctx")
     ap.add_argument("--calibrate-hbm", action="store_true", help="run the copy kernel of known traffic (for rocprofv3 --pmc)")
     ap.add_argument("--handover-probe", action="store_true", help="store/load cache-policy visibility probe between two workgroups")
     ap.add_argument("--placement", action="store_true", help="which XCD and CU the workgroups of a 128/256/512-workgroup launch land on")
@@ -615,6 +658,8 @@ def main():
         return run_gemv(args)
     if args.stack:
         return run_stack(args, ctx_list[0])
+    if args.stream_variants:
+        return run_stream_variants(args, ctx_list)
 
     sw = Sweep(ctx_list, n_q, args.layout, args.plain_workspace)
     layout_name = "head-major" if args.layout == 1 else "position-major"

@@ -31,6 +31,19 @@ int llmi_hip_probe_stream_read(const void* a, const void* b, size_t bytes_each, 
 int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, int32_t heads, int32_t workgroups_per_head,
                                     int32_t waves, int32_t tiles_in_flight, void* sink, void* stream);
 
+/* The decode kernel's K/V stream without its arithmetic, one feature at a time, on the decode kernel's own grid
+ * (kv_heads x splits workgroups, the KV head fastest; a head's 16-position tiles dealt to splits and wavefronts as the
+ * decode kernel deals them). `k`, `v`: caches of `positions` positions (a multiple of 16) of `kv_heads` heads x 256
+ * bytes in `kv_layout` (LLMI_KV_LAYOUT_*). (waves, tiles_in_flight) one of (4,2), (8,1), (8,2), (4,4). `mode`:
+ * 0 = ordinary non-temporal loads to registers; 1 = LDS-DMA loads into per-wavefront rings, whole rows per
+ * instruction; 2 = 1 with the K chunks swizzled by row & 7, exactly the decode kernel's requests; 3 = 2 with a pause
+ * of `pause` x 64 clocks (0..1024) after every tile has landed, standing for the arithmetic. `stagger` != 0: the
+ * splits start their walks at different tiles (the decode kernel's choice for some position-major lengths).
+ * Everything read is thrown away; `sink` (>= 4 bytes, device) is never written in practice. */
+int llmi_hip_probe_stream_tiles(const void* k, const void* v, int32_t positions, int32_t kv_heads, int32_t kv_layout, int32_t splits,
+                                int32_t waves, int32_t tiles_in_flight, int32_t mode, int32_t pause, int32_t stagger, void* sink,
+                                void* stream);
+
 /* dst[i] = src[i] for `bytes` bytes (a multiple of 16) with one plain kernel: reads `bytes`, writes `bytes`.
  * The known traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by. */
 int llmi_hip_probe_copy(const void* src, void* dst, size_t bytes, void* stream);

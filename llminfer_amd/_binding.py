@@ -138,6 +138,7 @@ SYMBOLS = {
     # include/llmi_hip_probes.h
     "llmi_hip_probe_stream_read": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
     "llmi_hip_probe_stream_read_rows": (ctypes.c_int, [c_void_p, c_void_p, c_i32, c_i32, c_i32, c_i32, c_i32, c_void_p, c_void_p]),
+    "llmi_hip_probe_stream_tiles": (ctypes.c_int, [c_void_p, c_void_p] + [c_i32] * 9 + [c_void_p, c_void_p]),
     "llmi_hip_probe_copy": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "llmi_hip_probe_block_pingpong": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "llmi_hip_strerror": (ctypes.c_char_p, [ctypes.c_int]),

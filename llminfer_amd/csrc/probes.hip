@@ -87,6 +87,94 @@ __global__ __launch_bounds__(NW * 64) void stream_read_rows_kernel(const char* _
     if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[0] = acc[0];
 }
 
+// The decode kernel's K/V stream without its arithmetic, one feature at a time: the same grid (KV head x split, the
+// KV head fastest), the same deal of 16-position tiles to splits and wavefronts, NSTAGE tiles in flight per wavefront.
+//   MODE 0: ordinary non-temporal loads to registers, a lane's 16 bytes at its own offset of the row (the floor kernel's way)
+//   MODE 1: LDS-DMA loads (global_load_lds_dwordx4 nt) into a per-wavefront ring, whole rows per instruction
+//   MODE 2: MODE 1 with the K chunks swizzled by row & 7 -- exactly what the decode kernel requests
+//   MODE 3: MODE 2 with a pause of `pause` x 64 clocks after every tile has landed: a wavefront that does its
+//           arithmetic is not requesting
+// `rs`: bytes between consecutive positions of one KV head (256 head-major, 256 x KV heads position-major);
+// `stagger`: the splits start their walks at different tiles (the decode kernel's STAGGER).
+__device__ __forceinline__ void probe_dma16(const char* base, uint32_t voff, uint32_t lds_off) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    const uint64_t sbase = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    const uint32_t slds = (uint32_t)__builtin_amdgcn_readfirstlane(lds_off);
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" :: "v"(voff), "s"(sbase), "{m0}"(slds) : "memory");
+}
+
+template <int NW, int NSTAGE, int MODE>
+__global__ __launch_bounds__(NW * 64) void stream_tiles_kernel(const char* __restrict__ k, const char* __restrict__ v, int tiles_per_head,
+                                                               int64_t head_bytes, uint32_t rs, int pause, int stagger, uint32_t* sink) {
+    __shared__ __attribute__((aligned(1024))) char smem[MODE == 0 ? 1024 : NW * NSTAGE * 8192];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n16 = lane & 15, kg = lane >> 4;
+    const int kvh = blockIdx.x, split = blockIdx.y, S = gridDim.y;
+    const int run = tiles_per_head / S, longer = tiles_per_head % S;
+    const int ntiles = run + (split < longer ? 1 : 0);
+    const int begin = split * run + min(split, longer);
+    const char* kb = k + kvh * head_bytes + (int64_t)begin * 16 * rs;
+    const char* vb = v + kvh * head_bytes + (int64_t)begin * 16 * rs;
+    const int n_my = wave < ntiles ? (ntiles - wave + NW - 1) / NW : 0;
+    const int rot = stagger ? min(split & 3, max(n_my - 1, 0)) : 0;
+    auto tile_of = [&](int i) {
+        int ii = i + rot;
+        if (ii >= n_my) ii -= n_my;
+        return wave + ii * NW;
+    };
+    const uint32_t k_row = kg * rs, col_lin = n16 * 16u;
+    const uint32_t k_col0 = MODE >= 2 ? (uint32_t)(n16 ^ kg) * 16u : col_lin;
+    const uint32_t k_col1 = MODE >= 2 ? (uint32_t)(n16 ^ (4 + kg)) * 16u : col_lin;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    if constexpr (MODE == 0) {
+        for (int i0 = 0; i0 < n_my; i0 += NSTAGE) {
+            u32x4 r[NSTAGE][8];
+#pragma unroll
+            for (int u = 0; u < NSTAGE; ++u) {
+                const uint32_t base = (uint32_t)tile_of(min(i0 + u, n_my - 1)) * 16u * rs + k_row + col_lin;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    r[u][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + base + j * 4 * rs));
+                    r[u][4 + j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb + base + j * 4 * rs));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < NSTAGE; ++u)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc ^= r[u][j];
+        }
+    } else {
+        const uint32_t ring = (uint32_t)(uintptr_t)(smem + wave * NSTAGE * 8192);
+        auto issue = [&](int i, int stage) {
+            const uint32_t base = (uint32_t)tile_of(i) * 16u * rs;
+            const uint32_t slot = ring + stage * 8192u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) probe_dma16(kb, base + k_row + j * 4u * rs + ((j & 1) ? k_col1 : k_col0), slot + j * 1024);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) probe_dma16(vb, base + k_row + j * 4u * rs + col_lin, slot + 4096 + j * 1024);
+        };
+        for (int s0 = 0; s0 < NSTAGE; ++s0)
+            if (s0 < n_my) issue(s0, s0);
+        int stage = 0;
+        for (int i = 0; i < n_my; ++i) {
+            const int newer = min(NSTAGE - 1, n_my - 1 - i);
+            if (newer <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else if (newer == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            else if (newer == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+            acc ^= *reinterpret_cast<const u32x4*>(smem + wave * NSTAGE * 8192 + stage * 8192 + lane * 16);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (i + NSTAGE < n_my) issue(i + NSTAGE, stage);
+            if constexpr (MODE == 3)
+                for (int p = 0; p < pause; ++p) __builtin_amdgcn_s_sleep(1);
+            stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
+        }
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[0] = acc[0];
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t n16) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
@@ -154,6 +242,19 @@ bool launch_stream(int inflight, dim3 grid, hipStream_t s, const char* a, const 
         case 1: hipLaunchKernelGGL((stream_read_kernel<NW, 1>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
         case 2: hipLaunchKernelGGL((stream_read_kernel<NW, 2>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
         case 4: hipLaunchKernelGGL((stream_read_kernel<NW, 4>), grid, dim3(NW * 64), 0, s, a, b, tiles, sink); return true;
+        default: return false;
+    }
+}
+
+template <int NW, int NSTAGE>
+bool launch_stream_tiles(int mode, dim3 grid, hipStream_t s, const char* k, const char* v, int tiles, int64_t head_bytes, uint32_t rs,
+                         int pause, int stagger, uint32_t* sink) {
+    const dim3 block(NW * 64);
+    switch (mode) {
+        case 0: hipLaunchKernelGGL((stream_tiles_kernel<NW, NSTAGE, 0>), grid, block, 0, s, k, v, tiles, head_bytes, rs, pause, stagger, sink); return true;
+        case 1: hipLaunchKernelGGL((stream_tiles_kernel<NW, NSTAGE, 1>), grid, block, 0, s, k, v, tiles, head_bytes, rs, pause, stagger, sink); return true;
+        case 2: hipLaunchKernelGGL((stream_tiles_kernel<NW, NSTAGE, 2>), grid, block, 0, s, k, v, tiles, head_bytes, rs, pause, stagger, sink); return true;
+        case 3: hipLaunchKernelGGL((stream_tiles_kernel<NW, NSTAGE, 3>), grid, block, 0, s, k, v, tiles, head_bytes, rs, pause, stagger, sink); return true;
         default: return false;
     }
 }
@@ -274,6 +375,33 @@ int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, 
         case 8: ok = launch_stream_rows<8>(tiles_in_flight, grid, s, pa, pb, tiles, row_bytes, ps); break;
         default: ok = false;
     }
+    if (!ok) return LLMI_ERR_INVALID_ARG;
+    return check_launch();
+}
+
+int llmi_hip_probe_stream_tiles(const void* k, const void* v, int32_t positions, int32_t kv_heads, int32_t kv_layout, int32_t splits,
+                                int32_t waves, int32_t tiles_in_flight, int32_t mode, int32_t pause, int32_t stagger, void* sink, void* stream) {
+    if (!k || !v || !sink) return LLMI_ERR_NULL_POINTER;
+    if (positions < 16 || positions % 16 != 0 || kv_heads < 1 || kv_heads > 1024) return LLMI_ERR_INVALID_ARG;
+    if (splits < 1 || splits > 65535 || splits > positions / 16) return LLMI_ERR_INVALID_ARG;
+    if (kv_layout != LLMI_KV_LAYOUT_POS_MAJOR && kv_layout != LLMI_KV_LAYOUT_HEAD_MAJOR) return LLMI_ERR_LAYOUT;
+    if (mode < 0 || mode > 3 || pause < 0 || pause > 1024) return LLMI_ERR_INVALID_ARG;
+    if (((uintptr_t)k | (uintptr_t)v) & 15u) return LLMI_ERR_ALIGNMENT;
+    const bool pm = kv_layout == LLMI_KV_LAYOUT_POS_MAJOR;
+    const uint32_t rs = pm ? (uint32_t)kv_heads * 256u : 256u;
+    const int64_t head_bytes = pm ? 256 : (int64_t)positions * 256;
+    if ((uint64_t)positions * rs > 0xffffffffull) return LLMI_ERR_INVALID_ARG;  // (32-bit offsets inside a head's run)
+    const dim3 grid((unsigned)kv_heads, (unsigned)splits);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const char* kp = static_cast<const char*>(k);
+    const char* vp = static_cast<const char*>(v);
+    uint32_t* ps = static_cast<uint32_t*>(sink);
+    const int tiles = positions / 16;
+    bool ok = false;
+    if (waves == 4 && tiles_in_flight == 2) ok = launch_stream_tiles<4, 2>(mode, grid, s, kp, vp, tiles, head_bytes, rs, pause, stagger, ps);
+    else if (waves == 8 && tiles_in_flight == 1) ok = launch_stream_tiles<8, 1>(mode, grid, s, kp, vp, tiles, head_bytes, rs, pause, stagger, ps);
+    else if (waves == 8 && tiles_in_flight == 2) ok = launch_stream_tiles<8, 2>(mode, grid, s, kp, vp, tiles, head_bytes, rs, pause, stagger, ps);
+    else if (waves == 4 && tiles_in_flight == 4) ok = launch_stream_tiles<4, 4>(mode, grid, s, kp, vp, tiles, head_bytes, rs, pause, stagger, ps);
     if (!ok) return LLMI_ERR_INVALID_ARG;
     return check_launch();
 }

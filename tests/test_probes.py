@@ -32,6 +32,23 @@ def test_stream_read_rows_rejects_bad_arguments():
     assert f(P, P + 4, 64, 8, 1, 4, 1, P, None) == B.STATUS["ALIGNMENT"]
 
 
+def test_stream_tiles_rejects_bad_arguments():
+    f = B.lib().llmi_hip_probe_stream_tiles
+    ok = dict(positions=64, kv_heads=8, kv_layout=1, splits=2, waves=4, inflight=2, mode=2, pause=0, stagger=0)
+
+    def call(k=P, v=P, sink=P, **over):
+        a = dict(ok, **over)
+        return f(k, v, a["positions"], a["kv_heads"], a["kv_layout"], a["splits"], a["waves"], a["inflight"], a["mode"], a["pause"],
+                 a["stagger"], sink, None)
+
+    assert call(k=None) == B.STATUS["NULL_POINTER"] and call(sink=None) == B.STATUS["NULL_POINTER"]
+    assert call(positions=0) == B.STATUS["INVALID_ARG"] and call(positions=65) == B.STATUS["INVALID_ARG"]
+    assert call(splits=5) == B.STATUS["INVALID_ARG"]        # more splits than tiles
+    assert call(kv_layout=2) == B.STATUS["LAYOUT"]
+    assert call(mode=4) == B.STATUS["INVALID_ARG"] and call(pause=-1) == B.STATUS["INVALID_ARG"]
+    assert call(k=P + 8) == B.STATUS["ALIGNMENT"]
+
+
 def test_copy_and_handover_reject_bad_arguments():
     lib = B.lib()
     assert lib.llmi_hip_probe_copy(None, P, 16, None) == B.STATUS["NULL_POINTER"]
@@ -82,6 +99,31 @@ def test_stream_probes_run_every_launch_shape(dev):
                                                       stream) == 0
     assert lib.llmi_hip_probe_stream_read(k.data_ptr(), v.data_ptr(), nbytes, 4, 3, 1, sink.data_ptr(), stream) == B.STATUS["INVALID_ARG"]
     assert lib.llmi_hip_probe_stream_read_rows(k.data_ptr(), v.data_ptr(), rows, heads, 4, 4, 3, sink.data_ptr(), stream) == B.STATUS["INVALID_ARG"]
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0
+
+
+@pytest.mark.gpu
+def test_stream_tiles_probe_runs_every_mode_and_shape(dev):
+    """Every mode, launch shape and layout of the stream-variants kernel on ragged tile counts: the launches succeed, the
+    sink stays untouched, and an unsupported (waves, tiles in flight) pair is refused."""
+    import torch
+    lib = B.lib()
+    positions, heads = 16 * 37, 8
+    nbytes = positions * heads * 256
+    k = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev)
+    v = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for layout in (0, 1):
+        for waves, inflight in ((4, 2), (8, 1), (8, 2), (4, 4)):
+            for mode in range(4):
+                for splits in (1, 3, 8, 37):
+                    for stagger in (0, 1):
+                        assert lib.llmi_hip_probe_stream_tiles(k.data_ptr(), v.data_ptr(), positions, heads, layout, splits, waves, inflight,
+                                                               mode, 2, stagger, sink.data_ptr(), stream) == 0
+    assert lib.llmi_hip_probe_stream_tiles(k.data_ptr(), v.data_ptr(), positions, heads, 1, 4, 2, 2, 0, 0, 0, sink.data_ptr(),
+                                           stream) == B.STATUS["INVALID_ARG"]
     torch.cuda.synchronize()
     assert int(sink.abs().sum()) == 0
 
