@@ -505,6 +505,94 @@ def run_calibrate_hbm(args):
     return 0
 
 
+def run_stack_timeline(args, ctx):
+    """Where a layer's time goes inside the resident launch (llmi_hip_mha_decode_append_stack): needs a build of the
+    library with the phase stamps compiled in,
+
+        python -m llminfer_amd.build --define LLMI_STACK_STAMPS=1 --only mha_stack.hip --output /tmp/libllmi_stamps.so
+        LLMI_HIP_LIBRARY=/tmp/libllmi_stamps.so python bench.py --stack-timeline --ctx 4096
+
+    which writes the 100 MHz clock at the phases of four layers (16 .. 19 of 36) into the workspace, 4 MiB in; this mode runs
+    the launch once after three warm-up launches and condenses the stamps. Times in us (ticks of 10 ns)."""
+    import numpy as np
+    import torch
+    from llminfer_amd import _binding as B
+    from llminfer_amd import ops
+    dev = torch.device("cuda:0")
+    L, n_q, D = 36, args.heads, HEAD_DIM
+    msl, pos, dim = ctx + 8, ctx, n_q * D
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+
+    def rnd(*shape, norm=True):
+        x = torch.randn(shape, generator=gen, device=dev)
+        if norm:
+            x = x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True))
+        return x.to(torch.bfloat16)
+
+    k, v = rnd(L * N_KV * msl, D).reshape(-1), rnd(L * N_KV * msl, D).reshape(-1)
+    q, kn, vn = rnd(L * n_q, D, norm=False).reshape(-1), rnd(L * N_KV, D, norm=False).reshape(-1), rnd(L * N_KV, D, norm=False).reshape(-1)
+    w = (1 + 0.02 * torch.randn(L * 2 * D, generator=gen, device=dev)).to(torch.bfloat16)
+    out = torch.zeros(L * dim, dtype=torch.bfloat16, device=dev)
+    sin_d, cos_d = ops.sincos_table(D, msl, dev)
+    ws = torch.zeros(max(ops.workspace_bytes(n_q, D, msl), 6 << 20) // 4, dtype=torch.float32, device=dev)
+    side = ops.workspace_side(ws)
+    kw = dict(layer_id=0, pos=pos, kv_dim=KV_DIM, kv_mul=n_q // N_KV, head_num=n_q, head_dim=D, max_seq_len=msl,
+              kv_layout=B.KV_LAYOUT_HEAD_MAJOR, workspace_side=side)
+
+    def run():
+        n = ops.mha_decode_append_stack(q, kn, vn, w, sin_d, cos_d, k, v, out, ws, layer_count=L, query_stride=dim, key_new_stride=KV_DIM,
+                                        value_new_stride=KV_DIM, norm_weight_stride=2 * D, output_stride=dim, **kw)
+        torch.cuda.synchronize()
+        return n
+
+    for _ in range(3):
+        run()
+    plan = ops.mha_plan(ops.make_mha_args(q, k, v, out, ws, **dict(kw, pos=pos - 1)))  # (the stack plans for the cached positions)
+    pad = ((-ws.data_ptr()) & 16383) if side else 0  # (the by-side layout starts on the next 16 KiB boundary)
+    first = (pad + (4 << 20)) // 4
+    ws[first:].zero_()
+    torch.cuda.synchronize()
+    if run() != 1:
+        print("bench.py: the one-launch form does not apply to this shape", file=sys.stderr)
+        return 1
+    S = plan.num_splits
+    grid = N_KV * S
+    st = ws[first:first + 4 * grid * 16].cpu().numpy().view(np.uint32).reshape(4, grid, 16).astype(np.int64)
+    if not st.any():
+        print("bench.py: no stamps found: build the library with --define LLMI_STACK_STAMPS=1 (see --help)", file=sys.stderr)
+        return 1
+    split = np.arange(grid) // N_KV
+    group = n_q // N_KV
+    merging = (split >= S - group) if S >= group else (split == S - 1)
+
+    def stats(x):
+        return {"min": round(float(x.min()) / 100, 2), "median": round(float(np.median(x)) / 100, 2), "max": round(float(x.max()) / 100, 2)}
+
+    layers = []
+    for l in range(1, 4):
+        t0 = st[l - 1, merging, 6].max()  # the last tag of the layer before
+        layers.append({
+            "layer": 16 + l,
+            "tags_seen_after_last_tag": stats(st[l, :, 0] - t0),
+            "operands_landed_after_tags_seen": stats(st[l, :, 1] - st[l, :, 0]),
+            "tiles_done_after_operands": stats(st[l, :, 8:12] - st[l, :, 1:2]),
+            "handed_over_after_tiles_done": stats(st[l, :, 3] - st[l, :, 2]),
+            "merging_records_in_after_own_hand_over": stats(st[l, merging, 4] - st[l, merging, 3]),
+            "merging_rows_read_back_after_records": stats(st[l, merging, 5] - st[l, merging, 4]),
+            "merging_tag_out_after_read_back": stats(st[l, merging, 6] - st[l, merging, 5]),
+            "layer_period": round(float(st[l, merging, 6].max() - t0) / 100, 2),
+        })
+    print(json.dumps({"metric": "phases of a layer inside the resident launch, us (100 MHz clock stamps of one launch)", "n_gpus": 1,
+                      "config": {"workload": "36 layers, %d Q / 8 KV heads, ctx %d + 1, %d splits; every figure over all %d workgroups (merging_*: "
+                                             "over the %d that merge a head)" % (n_q, ctx, S, grid, int(merging.sum()))},
+                      "note": "a stamp is a store: wavefront 0's own stamps add up to 0.4 us to its tile phase (its next tile wait also waits "
+                              "for the stamp's acknowledgement); the other wavefronts' tile times (tiles_done_after_operands covers all four) "
+                              "are undisturbed",
+                      "layers": layers}))
+    return 0
+
+
 STREAM_MODES = ["registers, linear", "LDS-DMA, linear", "LDS-DMA, K swizzled (the decode kernel's requests)",
                 "LDS-DMA, K swizzled, pause after every tile"]
 
@@ -609,6 +697,9 @@ def main():
                     help="time the automatic plan against forced single-pass / split plans at every --ctx")
     ap.add_argument("--stream-floor", action="store_true",
                     help="time a kernel that only reads the same K/V bytes, next to the decode kernel, at every --ctx")
+    ap.add_argument("--stack-timeline", action="store_true",
+                    help="phases of a layer inside the resident launch from in-kernel clock stamps; needs a library built with "
+                         "--define LLMI_STACK_STAMPS=1 (LLMI_HIP_LIBRARY), see run_stack_timeline")
     ap.add_argument("--stream-variants", action="store_true",
                     help="time the decode kernel's K/V stream without its arithmetic, one feature of the request pattern at a time, "
                          "in both cache layouts, at every --ctx")
@@ -660,6 +751,8 @@ def main():
         return run_stack(args, ctx_list[0])
     if args.stream_variants:
         return run_stream_variants(args, ctx_list)
+    if args.stack_timeline:
+        return run_stack_timeline(args, ctx_list[0])
 
     sw = Sweep(ctx_list, n_q, args.layout, args.plain_workspace)
     layout_name = "head-major" if args.layout == 1 else "position-major"
