@@ -36,6 +36,11 @@ int32_t llmi_hip_side_agreement(const int32_t* decisions, int32_t count, int32_t
  * out[0] = regions with an agreed side, out[1] = abstentions, out[2] = contradictions. */
 void llmi_hip_workspace_side_stats(uint64_t out[3]);
 
+/* The launcher's rule for the staggered walk of the split path (split s starts its walk s & mask tiles into each
+ * wavefront's sequence): the mask it would use for a cache in `kv_layout` whose splits' runs are `run_bytes` long
+ * (`ragged` != 0: some splits take one tile more); 0 = every split starts at its first tile. Makes no HIP call. */
+int32_t llmi_hip_stagger_mask(int32_t kv_layout, int64_t run_bytes, int32_t ragged);
+
 #ifdef __cplusplus
 }
 #endif

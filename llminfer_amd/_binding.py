@@ -147,6 +147,7 @@ SYMBOLS = {
     "llmi_hip_set_test_far_home": (c_i32, [c_i32]),
     "llmi_hip_side_from_pingpong": (c_i32, [ctypes.POINTER(ctypes.c_uint32)]),
     "llmi_hip_side_agreement": (c_i32, [ctypes.POINTER(c_i32), c_i32, ctypes.POINTER(c_i32)]),
+    "llmi_hip_stagger_mask": (c_i32, [c_i32, ctypes.c_int64, c_i32]),
     "llmi_hip_workspace_side_stats": (None, [ctypes.POINTER(ctypes.c_uint64)]),
 }
 

@@ -117,6 +117,25 @@ int spread_merge_min_splits(int group_pad) {
     return v ? v : group_pad >= 8 ? 16 : 32;
 }
 
+// Where the splits' runs start a multiple of 512 KiB apart, the workgroups of a KV head, walking in step, keep hitting
+// the same few memory channels; the splits then start their walks at different tiles (STAGGER kernels, split s rotated
+// by s & mask tiles of each wavefront's sequence).
+// Position-major, runs up to 1 MiB, mask 3. 32 Q / 8 KV heads, with : without: 9.44 : 10.54 us at 8192 positions
+// (512 KiB apart), level at 16384 (1 MiB); everywhere else the wrap-round only costs: 8.32 : 7.99 at 6144, 26.1 : 25.2
+// at 32768, 47.6 : 45.5 at 65536, level at 2048, 4096, 7168, 9216 ... 24576.
+// Head-major, runs from 1 MiB (up to 8 tiles above a multiple of 512 KiB count too: the position moves on by one per
+// token), mask 31. With : without, two layouts of the caches in memory each: 64 Q heads at 131072 positions 81.6 : 88.2
+// and 82.3 : 87.4 us, 32 Q heads 80.4 : 86.3 and 82.5 : 87.4; at 196608 123.3 : 126.8 and 125.7 : 130.2. Not at 65536
+// (512 KiB: 43.3 : 46.1 in one layout, 46.9 : 44.2 in the other), not between the multiples (163840: 108.8 : 100.7),
+// and no gain below (16384: 14.2 : 13.9). LLMI_HIP_STAGGER_MASK overrides the head-major mask (0 = never).
+int stagger_mask(int kv_layout, int64_t run_bytes, bool ragged) {
+    if (kv_layout == LLMI_KV_LAYOUT_POS_MAJOR)
+        return !ragged && run_bytes > 0 && run_bytes % (512 << 10) == 0 && run_bytes <= (1 << 20) ? 3 : 0;
+    static const int v = env_int("LLMI_HIP_STAGGER_MASK", 0, 255, -1);
+    if (v >= 0) return v;
+    return run_bytes >= (1 << 20) && run_bytes % (512 << 10) < 8 * 4096 ? 31 : 0;
+}
+
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }
 
 static int validate_mha(const llmi_mha_args* a) {
@@ -666,6 +685,10 @@ int llmi_hip_abi_version(void) { return LLMI_HIP_ABI_VERSION; }
 
 int32_t llmi_hip_set_test_far_home(int32_t mode) {
     return llmi::g_test_far_home.exchange(mode < 0 || mode > 2 ? 0 : mode, std::memory_order_relaxed);
+}
+
+int32_t llmi_hip_stagger_mask(int32_t kv_layout, int64_t run_bytes, int32_t ragged) {
+    return llmi::stagger_mask(kv_layout, run_bytes, ragged != 0);
 }
 
 int32_t llmi_hip_set_poll_limit(int32_t polls) {

@@ -67,6 +67,9 @@ constexpr bool by_side_variant(int group_pad, int waves) { return group_pad <= 8
 int read_poll_timeouts(unsigned long long* count);
 // Fewest splits at which the fused combine hands the heads of a KV head to different workgroups.
 int spread_merge_min_splits(int group_pad);
+// The mask of the staggered walk (KernelArgs::stagger) for splits whose runs are `run_bytes` long (the shorter ones,
+// when they differ by a tile: `ragged`).
+int stagger_mask(int kv_layout, int64_t run_bytes, bool ragged);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.
 int poll_limit();
 // Testing aid (llmi_hip_set_test_far_home): 1 = every split but the merging one, 2 = every second split stores into

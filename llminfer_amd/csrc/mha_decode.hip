@@ -184,7 +184,7 @@ static int fill_kernel_args(const llmi_mha_args& args, const llmi_mha_plan& plan
     ka.seq_len = args.pos + 1;
     ka.spread_merge = plan.num_splits >= spread_merge_min_splits(plan.group_pad);
     ka.max_polls = poll_limit();
-    ka.stagger = false;  // (decided below, once the runs of the splits are known)
+    ka.stagger = 0;  // (decided below, once the runs of the splits are known)
     ka.group = args.kv_mul;
     ka.n_q = args.head_num;
     ka.num_splits = plan.num_splits;
@@ -193,14 +193,8 @@ static int fill_kernel_args(const llmi_mha_args& args, const llmi_mha_plan& plan
         const int tiles = (cached + kTile - 1) / kTile;
         ka.tiles_run = tiles / plan.num_splits;
         ka.tiles_longer = tiles % plan.num_splits;
-        // Position-major layout: when the splits' runs start a multiple of 512 KiB apart (up to 1 MiB) the workgroups
-        // of a KV head, walking in step, keep hitting the same few memory channels; the splits then start their walks
-        // at different tiles (STAGGER). 32 Q / 8 KV heads, with : without: 9.44 : 10.54 us at 8192 positions (512 KiB
-        // apart), level at 16384 (1 MiB); everywhere else the wrap-round only costs: 8.32 : 7.99 at 6144, 26.1 : 25.2 at
-        // 32768, 47.6 : 45.5 at 65536, level at 2048, 4096, 7168, 9216 ... 24576.
-        const int64_t run_bytes = (int64_t)ka.tiles_run * kTile * ka.row_stride * 2;
-        ka.stagger = args.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR && ka.tiles_longer == 0 && run_bytes > 0 &&
-                     run_bytes % (512 << 10) == 0 && run_bytes <= (1 << 20);
+        // (where the splits' runs start a multiple of 512 KiB apart the splits start their walks at different tiles)
+        ka.stagger = stagger_mask(args.kv_layout, (int64_t)ka.tiles_run * kTile * ka.row_stride * 2, ka.tiles_longer != 0);
     }
     ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
     if (append) {

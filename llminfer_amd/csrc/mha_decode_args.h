@@ -23,7 +23,7 @@ struct KernelArgs {
     int32_t seq_len;
     int32_t tiles_run, tiles_longer;  // tiles per split and how many splits take one more (position known on the host)
     int32_t max_polls;             // polls of the fused combine before it gives up and writes NaN
-    bool stagger;                  // walk the tiles of a split from a split-dependent starting point (plain variant only)
+    int32_t stagger;               // != 0: split s starts its walk (s & stagger) tiles into each wavefront's sequence (STAGGER kernels)
     int32_t group;        // query heads per KV head
     int32_t n_q;          // query heads
     int32_t num_splits;

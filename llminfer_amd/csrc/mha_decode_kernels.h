@@ -312,13 +312,14 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
 
     // Wave w owns tiles w, w+NW, ...: NSTAGE of them are always in flight.
     const int n_my = wave < ntiles ? (ntiles - wave + NW - 1) / NW : 0;
-    // STAGGER (position-major layout): the splits of a head walk their tiles from different starting
-    // points (split s starts s mod 4 tiles into its wave's sequence and wraps round), so that
-    // workgroups running in step do not all sit at the same offset of their runs. At 8192 positions
-    // the runs start exactly 512 KiB apart and walking them in step costs 1.7 us of 13.6. The
-    // head-major layout gains nothing from it and the bookkeeping costs 0.08 us per call, so it
-    // is compiled in only where it is used.
-    const int rot = STAGGER ? min(split & 3, max(n_my - 1, 0)) : 0;
+    // STAGGER: the splits of a head walk their tiles from different starting points (split s starts
+    // s & a.stagger tiles into its wave's sequence and wraps round), so that workgroups running in
+    // step do not all sit at the same offset of their runs. Where the runs start a multiple of 512 KiB
+    // apart, walking them in step keeps hitting the same few memory channels: position-major, 8192
+    // positions, 1.7 us of 13.6; head-major, 131072 positions (runs of 1 MiB), 6 us of 87. Elsewhere it
+    // gains nothing or loses, and the bookkeeping costs 0.08 us per call, so the host asks for it by
+    // length and it is compiled in only where it is used.
+    const int rot = STAGGER ? min(split & a.stagger, max(n_my - 1, 0)) : 0;
     auto tile_of = [&](int i) {
         if constexpr (!STAGGER) return wave + i * NW;
         int ii = i + rot;
@@ -1059,6 +1060,8 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
         if (ka.by_side) {
             if (append) {
                 if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else if (ka.stagger)
+                    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, true, true>), grid, dim3(NW * 64), 0, stream, ka);
                 else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
             } else {
                 if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
@@ -1071,6 +1074,8 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
     }
     if (append) {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else if (ka.stagger && ka.num_splits > 1)
+            hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
     } else {
         if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);

@@ -111,14 +111,19 @@ __global__ __launch_bounds__(NW * 64) void stream_tiles_kernel(const char* __res
     __shared__ __attribute__((aligned(1024))) char smem[MODE == 0 ? 1024 : NW * NSTAGE * 8192];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n16 = lane & 15, kg = lane >> 4;
-    const int kvh = blockIdx.x, split = blockIdx.y, S = gridDim.y;
+    // (stagger bit 1: the grid has the splits fastest -- consecutive workgroups read consecutive runs of one head --
+    // instead of the decode kernel's KV heads fastest)
+    const bool splits_fastest = (stagger & 2) != 0;
+    const int rot_mask = (stagger & 1) ? 3 : (stagger >> 2);  // (bits 2 and up: another mask for the rotation)
+    const int kvh = splits_fastest ? blockIdx.y : blockIdx.x, split = splits_fastest ? blockIdx.x : blockIdx.y;
+    const int S = splits_fastest ? gridDim.x : gridDim.y;
     const int run = tiles_per_head / S, longer = tiles_per_head % S;
     const int ntiles = run + (split < longer ? 1 : 0);
     const int begin = split * run + min(split, longer);
     const char* kb = k + kvh * head_bytes + (int64_t)begin * 16 * rs;
     const char* vb = v + kvh * head_bytes + (int64_t)begin * 16 * rs;
     const int n_my = wave < ntiles ? (ntiles - wave + NW - 1) / NW : 0;
-    const int rot = stagger ? min(split & 3, max(n_my - 1, 0)) : 0;
+    const int rot = min(split & rot_mask, max(n_my - 1, 0));
     auto tile_of = [&](int i) {
         int ii = i + rot;
         if (ii >= n_my) ii -= n_my;
@@ -391,7 +396,8 @@ int llmi_hip_probe_stream_tiles(const void* k, const void* v, int32_t positions,
     const uint32_t rs = pm ? (uint32_t)kv_heads * 256u : 256u;
     const int64_t head_bytes = pm ? 256 : (int64_t)positions * 256;
     if ((uint64_t)positions * rs > 0xffffffffull) return LLMI_ERR_INVALID_ARG;  // (32-bit offsets inside a head's run)
-    const dim3 grid((unsigned)kv_heads, (unsigned)splits);
+    if (stagger < 0 || stagger > 255) return LLMI_ERR_INVALID_ARG;
+    const dim3 grid = (stagger & 2) ? dim3((unsigned)splits, (unsigned)kv_heads) : dim3((unsigned)kv_heads, (unsigned)splits);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const char* kp = static_cast<const char*>(k);
     const char* vp = static_cast<const char*>(v);

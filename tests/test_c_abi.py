@@ -383,6 +383,37 @@ def test_environment_overrides_of_the_dispatch():
     assert run(LLMI_HIP_NUM_SPLITS="junk", LLMI_HIP_SINGLE_PASS_MAX="-3") == run()
 
 
+def test_stagger_rule_of_the_split_path():
+    """Which lengths get the staggered walk: position-major where the splits' runs are exactly 512 KiB or 1 MiB,
+    head-major from 1 MiB at (or a few tiles above) a multiple of 512 KiB; LLMI_HIP_STAGGER_MASK overrides the
+    head-major mask only (read once per process: a child process per setting)."""
+    m = B.lib().llmi_hip_stagger_mask
+    K = 1 << 10
+    # position-major: 32 splits of 8192 positions x 2 KiB rows = 512 KiB each
+    assert m(B.KV_LAYOUT_POS_MAJOR, 512 * K, 0) == 3 and m(B.KV_LAYOUT_POS_MAJOR, 1024 * K, 0) == 3
+    assert m(B.KV_LAYOUT_POS_MAJOR, 512 * K, 1) == 0 and m(B.KV_LAYOUT_POS_MAJOR, 2048 * K, 0) == 0
+    assert m(B.KV_LAYOUT_POS_MAJOR, 384 * K, 0) == 0 and m(B.KV_LAYOUT_POS_MAJOR, 0, 0) == 0
+    # head-major: 131072 positions in 32 splits = 1 MiB runs; 196608 = 1.5 MiB; 65536 = 512 KiB; 163840 = 1.25 MiB
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K, 0) == 31 and m(B.KV_LAYOUT_HEAD_MAJOR, 1536 * K, 0) == 31
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K + 7 * 4096, 1) == 31  # the position has moved on by some tokens
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K + 8 * 4096, 1) == 0
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 512 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 1280 * K, 0) == 0
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 256 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 0, 0) == 0
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from llminfer_amd import _binding as B\n"
+            "m = B.lib().llmi_hip_stagger_mask\n"
+            "print(m(1, 1 << 20, 0), m(1, 256 << 10, 0), m(0, 512 << 10, 0), m(0, 2 << 20, 0))\n" % ROOT)
+
+    def run(**env):
+        e = dict(os.environ, **env)
+        return subprocess.run([sys.executable, "-c", code], check=True, stdout=subprocess.PIPE, text=True, env=e, cwd=ROOT).stdout.split()
+
+    assert run() == ["31", "0", "3", "0"]
+    assert run(LLMI_HIP_STAGGER_MASK="0") == ["0", "0", "3", "0"]
+    assert run(LLMI_HIP_STAGGER_MASK="7") == ["7", "7", "3", "0"]
+    assert run(LLMI_HIP_STAGGER_MASK="junk") == run()
+
+
 def test_side_decision_from_injected_timings():
     """The decision behind llmi_hip_mha_workspace_side as a pure function of the ping-pong probe's result words:
     clear cases, noise below the threshold, ties, pairs that lost a number or did not share an XCD, a side of the

@@ -268,6 +268,37 @@ def test_position_major_staggered_walk(oracle, dev, ctx, splits, waves):
     assert plan.num_splits > 1 and tiles // plan.num_splits >= 2 * plan.waves_per_group  # two or more tiles per wave
 
 
+def test_head_major_staggered_walk_forced(dev):
+    """The staggered walk of the head-major layout, which the launcher's rule only picks from 1 MiB runs on, forced on
+    small shapes (LLMI_HIP_STAGGER_MASK is read once per process: a child process): ragged runs, one to eight
+    wavefronts, more rotation than a wavefront has tiles, the append variant, by-side and plain workspace; every
+    result is the oracle's."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "import torch, oracle\n"
+        "from llminfer_amd import _binding as B, synth\n"
+        "from helpers import assert_parity, assert_tap_parity, run_hip, run_oracle\n"
+        "oracle.lib(); dev = torch.device('cuda:0')\n"
+        "assert B.lib().llmi_hip_stagger_mask(B.KV_LAYOUT_HEAD_MAJOR, 4096, 1) == 7\n"
+        "n = 0\n"
+        "for n_q, ctx, splits, waves, side in ((32, 4096, 0, 0, 'measure'), (32, 5003, 7, 4, 0), (32, 1000, 3, 1, 0), (32, 3001, 5, 2, 0x55555555),\n"
+        "                                      (64, 2049, 4, 8, 0xaaaaaaaa), (16, 700, 2, 4, 0), (8, 6000, 16, 4, 'measure')):\n"
+        "    case = synth.make_case(29 + n, ctx=ctx, n_q=n_q, n_kv=8)\n"
+        "    ref = run_oracle(oracle, case)\n"
+        "    kw = dict(force_path=B.PATH_SPLIT_FUSED, num_splits=splits, waves_per_group=waves) if splits else {}\n"
+        "    got16, got32, plan = run_hip(case, dev, kv_layout=B.KV_LAYOUT_HEAD_MAJOR, want_plan=True, workspace_side=side, **kw)\n"
+        "    assert plan.num_splits > 1\n"
+        "    assert_parity(got16, ref, 'staggered %%d/%%d/%%d/%%d' %% (n_q, ctx, splits, waves)); assert_tap_parity(got32, ref, 'tap'); n += 1\n"
+        "print('ok', n)\n" % (root, os.path.join(root, "tests")))
+    res = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=root,
+                         env=dict(os.environ, LLMI_HIP_STAGGER_MASK="7"), timeout=280)
+    assert res.returncode == 0 and "ok 7" in res.stdout, res.stdout[-3000:]
+
+
 def test_qwen3_32b_head_layout_at_128k(oracle, dev):
     """64 Q / 8 KV heads at ctx 131072 (512 MiB of K and V, seed 5) at full size against the oracle:
     the dispatcher's plan (fused combine, one workgroup per CU, 8 waves), the fused combine at the
