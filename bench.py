@@ -614,7 +614,7 @@ def run_stream_variants(args, ctx_list):
             decode_us = sw.us_per_call(lambda f, n: sw.enqueue([ctx], f, n), reps=3, replays=40, steps=n_slices(ctx))
             row = {"ctx": ctx, "layout": "head-major" if layout == 1 else "position-major", "splits": 32, "waves": waves,
                    "tiles_in_flight": inflight, "decode_us": round(decode_us, 2), "variants": []}
-            for mode, pause, stagger in ((0, 0, 0), (1, 0, 0), (2, 0, 0), (3, 4, 0), (3, 8, 0), (3, 16, 0), (0, 0, 2), (2, 0, 2), (2, 0, 1), (2, 0, 3)):
+            for mode, pause, stagger in ((0, 0, 0), (1, 0, 0), (2, 0, 0), (3, 4, 0), (3, 8, 0), (3, 16, 0), (0, 0, 2), (2, 0, 2), (2, 0, 1), (2, 0, 4 * 31), (2, 0, 2 + 4 * 31)):
                 def enq(first, n):
                     for st in range(first, first + n):
                         off = sw.regions[(ctx, st % n_slices(ctx))] * 2
@@ -622,7 +622,7 @@ def run_stream_variants(args, ctx_list):
                                       stagger, sw.sink.data_ptr(), sw.stream.cuda_stream), "llmi_hip_probe_stream_tiles")
                 us = sw.us_per_call(enq, reps=3, replays=40, steps=n_slices(ctx))
                 row["variants"].append({"mode": STREAM_MODES[mode] + (" (%d x 64 clocks)" % pause if mode == 3 else "") +
-                                                (", staggered walk" if stagger & 1 else "") +
+                                                (", staggered walk (mask %d)" % (3 if stagger & 1 else stagger >> 2) if stagger & ~2 else "") +
                                                 (", splits fastest in the grid" if stagger & 2 else ""),
                                         "us": round(us, 2), "TBps": round(2 * ctx * KV_DIM * 2 / us / 1e6, 3)})
             rows.append(row)

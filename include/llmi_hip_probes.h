@@ -37,9 +37,10 @@ int llmi_hip_probe_stream_read_rows(const void* a, const void* b, int32_t rows, 
  * bytes in `kv_layout` (LLMI_KV_LAYOUT_*). (waves, tiles_in_flight) one of (4,2), (8,1), (8,2), (4,4). `mode`:
  * 0 = ordinary non-temporal loads to registers; 1 = LDS-DMA loads into per-wavefront rings, whole rows per
  * instruction; 2 = 1 with the K chunks swizzled by row & 7, exactly the decode kernel's requests; 3 = 2 with a pause
- * of `pause` x 64 clocks (0..1024) after every tile has landed, standing for the arithmetic. `stagger` (0..3), bit 0:
- * the splits start their walks at different tiles (the decode kernel's choice for some position-major lengths);
- * bit 1: the grid is splits x kv_heads with the split fastest (consecutive workgroups read consecutive runs of a head).
+ * of `pause` x 64 clocks (0..1024) after every tile has landed, standing for the arithmetic. `stagger` (0..255):
+ * split s starts its walk s & mask tiles into each wavefront's sequence, mask = 3 if bit 0 is set, else stagger >> 2
+ * (the decode kernel's choice for some lengths: 3 position-major, 31 head-major); bit 1: the grid is splits x kv_heads
+ * with the split fastest (consecutive workgroups read consecutive runs of a head), not the decode kernel's order.
  * Everything read is thrown away; `sink` (>= 4 bytes, device) is never written in practice. */
 int llmi_hip_probe_stream_tiles(const void* k, const void* v, int32_t positions, int32_t kv_heads, int32_t kv_layout, int32_t splits,
                                 int32_t waves, int32_t tiles_in_flight, int32_t mode, int32_t pause, int32_t stagger, void* sink,

@@ -46,6 +46,7 @@ def test_stream_tiles_rejects_bad_arguments():
     assert call(splits=5) == B.STATUS["INVALID_ARG"]        # more splits than tiles
     assert call(kv_layout=2) == B.STATUS["LAYOUT"]
     assert call(mode=4) == B.STATUS["INVALID_ARG"] and call(pause=-1) == B.STATUS["INVALID_ARG"]
+    assert call(stagger=-1) == B.STATUS["INVALID_ARG"] and call(stagger=256) == B.STATUS["INVALID_ARG"]
     assert call(k=P + 8) == B.STATUS["ALIGNMENT"]
 
 
@@ -119,7 +120,7 @@ def test_stream_tiles_probe_runs_every_mode_and_shape(dev):
         for waves, inflight in ((4, 2), (8, 1), (8, 2), (4, 4)):
             for mode in range(4):
                 for splits in (1, 3, 8, 37):
-                    for stagger in (0, 1):
+                    for stagger in (0, 1, 2, 4 * 31, 2 + 4 * 7):  # none, mask 3, split-fastest grid, mask 31, both
                         assert lib.llmi_hip_probe_stream_tiles(k.data_ptr(), v.data_ptr(), positions, heads, layout, splits, waves, inflight,
                                                                mode, 2, stagger, sink.data_ptr(), stream) == 0
     assert lib.llmi_hip_probe_stream_tiles(k.data_ptr(), v.data_ptr(), positions, heads, 1, 4, 2, 2, 0, 0, 0, sink.data_ptr(),
