@@ -477,6 +477,19 @@ def dispatch_rows(sw, ctx_list):
     return rows
 
 
+def own_process_line(flags, timeout_s=150):
+    """The JSON line of `bench.py <flags>` run as a child process (this process keeps the GPU; the child gets its own
+    context and allocator state), or None if it fails."""
+    import subprocess
+    try:
+        res = subprocess.run([sys.executable, os.path.abspath(__file__)] + flags, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
+                             text=True, timeout=timeout_s, cwd=ROOT)
+        lines = [l for l in res.stdout.splitlines() if l.startswith("{")]
+        return json.loads(lines[-1]) if res.returncode == 0 and lines else None
+    except (subprocess.SubprocessError, OSError, ValueError):
+        return None
+
+
 def per_ctx_rows(sw, ctx_list, replays):
     rows = []
     for ctx in ctx_list:
@@ -887,6 +900,15 @@ def main():
                                   stream_floor_us=f5["us"], floor_ratio=round(f5["us"] / r5["us_per_layer"], 3))
             del sw5
             torch.cuda.empty_cache()
+            # The same workload as the driver-style run of a process of its own (`bench.py --heads 64 --ctx 131072`), whose
+            # arena is the first thing that process allocates: at this length the figure depends on where the two caches lie
+            # (the splits' runs are exactly 1 MiB long and resonate with the memory channels), so both are reported.
+            own = own_process_line(["--heads", "64", "--ctx", "131072", "--no-extras", "--no-cpu-baseline", "--steps", "64", "--warmup", "8"])
+            if own is not None:
+                result["cfg5"]["own_process"] = {"us_per_layer": own["roofline"]["avg_launch_us"], "frac_peak": own["roofline"]["frac"],
+                                                 "command": "python bench.py --heads 64 --ctx 131072 --no-extras --no-cpu-baseline --steps 64 --warmup 8",
+                                                 "note": "the same kernel and workload with the arena allocated first in a fresh process; "
+                                                         "us_per_layer above is this process's arena, allocated after three others were freed"}
             # BASELINE config 4: 36 layers at ctx 4096 + 1 new token, fused QK-Norm + RoPE + append, one HIP graph per token
             ns = argparse.Namespace(stack=36, heads=32, layout=1, stack_mode=5, stack_follow_pos=False, steps=200, warmup=20)
             r4 = stack_result(ns, 4096)
