@@ -481,6 +481,10 @@ def own_process_line(flags, timeout_s=150):
     """The JSON line of `bench.py <flags>` run as a child process (this process keeps the GPU; the child gets its own
     context and allocator state), or None if it fails."""
     import subprocess
+    # (not under a profiler: its preloaded library has the GPU open before a program starts, and a process in that
+    # state must not be replaced by another program, which is what starting a child amounts to)
+    if any(k.startswith(("ROCP", "ROCPROF")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", ""):
+        return None
     try:
         res = subprocess.run([sys.executable, os.path.abspath(__file__)] + flags, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
                              text=True, timeout=timeout_s, cwd=ROOT)
