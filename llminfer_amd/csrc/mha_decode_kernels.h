@@ -472,7 +472,15 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     }
 
     int stage = 0;
+#if LLMI_TIMING_BARRIER_PER_TILE
+    // (measurement only: what a scheme in which the wavefronts of a workgroup share every tile would pay for having to
+    // agree, tile by tile, that a slot may be refilled -- a workgroup barrier per tile, every wavefront the same number)
+    for (int i = 0; i < (ntiles + NW - 1) / NW; ++i) {
+        __syncthreads();
+        if (i >= n_my) continue;
+#else
     for (int i = 0; i < n_my; ++i) {
+#endif
         TileRegs r;
         wait_tiles_in_flight(min(NSTAGE - 1, n_my - 1 - i));
         read_tile(stage, r);

@@ -54,6 +54,10 @@ constexpr int kCacheDevice = 16;
 // 0: by the workgroup of the last split, a wavefront each. Kept for the side-by-side measurement.
 #define LLMI_SPREAD_MERGE 1
 #endif
+#ifndef LLMI_TIMING_BARRIER_PER_TILE
+// 1: a workgroup barrier in front of every tile of the decode kernel's loop (timing only: results unchanged, just slower).
+#define LLMI_TIMING_BARRIER_PER_TILE 0
+#endif
 #ifndef LLMI_PV_VALU
 // 1: the probability x value product runs on the vector ALU (fp32 multiply-adds with the
 // probabilities broadcast by DPP, the structure of the reference's inner loop,
