@@ -330,6 +330,9 @@ def run_stack(args, ctx):
     return 0
 
 
+SETTLE_MS = 40.0
+
+
 class Sweep:
     """Decode-attention calls over rotating KV slices, captured into HIP graphs and timed with HIP events."""
 
@@ -412,8 +415,13 @@ class Sweep:
         """Best (or, stat="all", every one) of `reps` batches of graph replays (a graph of `steps` steps), us per call."""
         g = self.capture(enqueue_fn, steps)
         scale = max(1, steps // SLICES)
-        self.time_replays([(g, max(1, 8 // scale))])
         n = max(1, (replays or 40) // scale)
+        # Untimed replays first, SETTLE_MS of them: after a pause (allocation, capture, host work) the device needs some
+        # ten milliseconds of the same load before its clocks have settled -- 64 Q heads at 131072 positions read 84.5 us
+        # per call in the first 10 ms, 83.3 after 20 ms and 80.8 from 40 ms on, also in short batches from then on.
+        spent = self.time_replays([(g, max(1, 8 // scale))])
+        while spent < SETTLE_MS:
+            spent += max(self.time_replays([(g, n)]), 0.05)
         samples = [self.time_replays([(g, n)]) * 1e3 / (n * steps * calls_per_step) for _ in range(reps)]
         return samples if stat == "all" else min(samples)
 
@@ -422,10 +430,17 @@ class Sweep:
 FLOOR_CONFIGS = [(256, 4, 2), (256, 8, 2), (512, 4, 2), (256, 4, 4), (512, 8, 1), (1024, 4, 1), (512, 4, 4), (256, 8, 4)]
 
 
-def stream_floor(sw, ctx_list, configs=FLOOR_CONFIGS):
+# ... and of the decode kernel's own grid (8 KV heads x 32 splits, LDS-DMA loads), with the splits' walks staggered by
+# split & mask tiles: (waves, tiles in flight, mask). Workgroups that walk their runs in step feel the resonances of the
+# request pattern with the memory channels; these do not, and are often the faster stream.
+FLOOR_STAGGERED = [(4, 2, 7), (4, 2, 31), (8, 1, 31)]
+
+
+def stream_floor(sw, ctx_list, configs=FLOOR_CONFIGS, staggered=FLOOR_STAGGERED):
     """Per context: the fastest stream-only launch (same K/V bytes read once and thrown away, same graph-replay
-    timing as the decode figures) over a handful of launch shapes."""
+    timing as the decode figures) over a handful of launch shapes and walks."""
     rows = []
+    probe_tiles = sw.B.lib().llmi_hip_probe_stream_tiles
     for ctx in ctx_list:
         best = None
         for wg, waves, inflight in configs:
@@ -434,11 +449,23 @@ def stream_floor(sw, ctx_list, configs=FLOOR_CONFIGS):
                 continue
             us = sw.us_per_call(lambda f, n: sw.enqueue_floor([ctx], f, n, wg, waves, inflight), reps=2, steps=n_slices(ctx))
             if best is None or us < best[0]:
-                best = (us, wg, waves, inflight)
-        us, wg, waves, inflight = best
+                best = (us, wg, waves, inflight, 0)
+        for waves, inflight, mask in staggered:
+            if ctx // 16 < 32 * waves * 2:  # (fewer than two tiles per wavefront: nothing to stagger)
+                continue
+
+            def enq(first, n, waves=waves, inflight=inflight, mask=mask):
+                for st in range(first, first + n):
+                    off = sw.regions[(ctx, st % n_slices(ctx))] * 2
+                    sw.B.check(probe_tiles(sw.k.data_ptr() + off, sw.v.data_ptr() + off, ctx, N_KV, sw.layout, 32, waves, inflight, 1, 0,
+                                           4 * mask, sw.sink.data_ptr(), sw.stream.cuda_stream), "llmi_hip_probe_stream_tiles")
+            us = sw.us_per_call(enq, reps=2, steps=n_slices(ctx))
+            if us < best[0]:
+                best = (us, 32 * N_KV, waves, inflight, mask)
+        us, wg, waves, inflight, mask = best
         gbs = 2 * ctx * KV_DIM * 2 / (us * 1e-6) / 1e9
         rows.append({"ctx": ctx, "us": round(us, 3), "GBps": round(gbs, 1), "frac_peak": round(gbs / HBM_PEAK_GBS, 4),
-                     "workgroups": wg, "waves": waves, "tiles_in_flight": inflight})
+                     "workgroups": wg, "waves": waves, "tiles_in_flight": inflight, "stagger_mask": mask})
     return rows
 
 
@@ -898,7 +925,7 @@ def main():
             torch.cuda.empty_cache()
             # BASELINE config 5: 64 Q / 8 KV heads at ctx 131072 (512 MiB of K and V per call)
             sw5 = Sweep([131072], 64, 1)
-            r5 = per_ctx_rows(sw5, [131072], 10)[0]
+            r5 = per_ctx_rows(sw5, [131072], 40)[0]  # (batches of 27 ms: shorter ones read 3 us more, the clocks have not settled)
             f5 = stream_floor(sw5, [131072], FLOOR_CONFIGS[:4])[0]
             result["cfg5"] = dict(r5, workload="64 Q / 8 KV heads, ctx 131072, head-major, graph replays over %d KV slices" % SLICES,
                                   stream_floor_us=f5["us"], floor_ratio=round(f5["us"] / r5["us_per_layer"], 3))
