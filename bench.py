@@ -331,6 +331,8 @@ def run_stack(args, ctx):
 
 
 SETTLE_MS = 40.0
+SETTLE_FIRST_MS = 600.0
+MIN_GRAPH_STEPS = 64
 
 
 class Sweep:
@@ -348,6 +350,7 @@ class Sweep:
         self.ws = torch.empty(ops.workspace_bytes(n_q, HEAD_DIM, max(self.ctx_list)) // 4, dtype=torch.float32, device=self.dev)
         self.sink = torch.zeros(64, dtype=torch.int32, device=self.dev)
         self.stream = torch.cuda.Stream()
+        self.settled = False  # (no figure taken on this arena yet: see us_per_call)
         self.decode = B.lib().llmi_hip_mha_decode
         # Set-up, once per workspace allocation, like an engine would do it: which 8 KiB blocks of the workspace lie
         # near which side of the package (the fused combine keeps its hand-over data in near memory then).
@@ -413,14 +416,22 @@ class Sweep:
 
     def us_per_call(self, enqueue_fn, calls_per_step=1, reps=3, replays=None, steps=SLICES, stat="best"):
         """Best (or, stat="all", every one) of `reps` batches of graph replays (a graph of `steps` steps), us per call."""
+        # At least MIN_GRAPH_STEPS calls per graph (the slices taken in turn, several times round): between two replays
+        # of a graph the device idles for some microseconds, which a decode step pays once per token, not once per layer
+        # -- with 8 calls per graph a call at 32768 positions reads 23.2 us, with 64 of them 22.6.
+        steps = max(steps, MIN_GRAPH_STEPS)
         g = self.capture(enqueue_fn, steps)
         scale = max(1, steps // SLICES)
         n = max(1, (replays or 40) // scale)
-        # Untimed replays first, SETTLE_MS of them: after a pause (allocation, capture, host work) the device needs some
-        # ten milliseconds of the same load before its clocks have settled -- 64 Q heads at 131072 positions read 84.5 us
-        # per call in the first 10 ms, 83.3 after 20 ms and 80.8 from 40 ms on, also in short batches from then on.
+        # Untimed replays first. After a pause (allocation, capture, host work) the device needs some ten milliseconds of
+        # the same load before its clocks have settled (SETTLE_MS, before every figure); after the seconds of other work
+        # and the allocation that precede a new arena it runs 4-5 % slow for a third of a second -- 64 Q heads at 131072
+        # positions: 84.5 us per call for 340-390 ms, 80.0 from then on; 32 Q heads at 32768: 24.25, then 23.2 --, so
+        # the first figure taken on an arena waits SETTLE_FIRST_MS.
         spent = self.time_replays([(g, max(1, 8 // scale))])
-        while spent < SETTLE_MS:
+        target = SETTLE_MS if self.settled else SETTLE_FIRST_MS
+        self.settled = True
+        while spent < target:
             spent += max(self.time_replays([(g, n)]), 0.05)
         samples = [self.time_replays([(g, n)]) * 1e3 / (n * steps * calls_per_step) for _ in range(reps)]
         return samples if stat == "all" else min(samples)
@@ -502,23 +513,6 @@ def dispatch_rows(sw, ctx_list):
                      "best_forced": best, "best_forced_us": round(med[best], 2), "auto_over_best": round(auto / med[best], 3),
                      "forced_us": {k2: round(v2, 2) for k2, v2 in med.items()}})
     return rows
-
-
-def own_process_line(flags, timeout_s=150):
-    """The JSON line of `bench.py <flags>` run as a child process (this process keeps the GPU; the child gets its own
-    context and allocator state), or None if it fails."""
-    import subprocess
-    # (not under a profiler: its preloaded library has the GPU open before a program starts, and a process in that
-    # state must not be replaced by another program, which is what starting a child amounts to)
-    if any(k.startswith(("ROCP", "ROCPROF")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", ""):
-        return None
-    try:
-        res = subprocess.run([sys.executable, os.path.abspath(__file__)] + flags, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
-                             text=True, timeout=timeout_s, cwd=ROOT)
-        lines = [l for l in res.stdout.splitlines() if l.startswith("{")]
-        return json.loads(lines[-1]) if res.returncode == 0 and lines else None
-    except (subprocess.SubprocessError, OSError, ValueError):
-        return None
 
 
 def per_ctx_rows(sw, ctx_list, replays):
@@ -925,21 +919,12 @@ def main():
             torch.cuda.empty_cache()
             # BASELINE config 5: 64 Q / 8 KV heads at ctx 131072 (512 MiB of K and V per call)
             sw5 = Sweep([131072], 64, 1)
-            r5 = per_ctx_rows(sw5, [131072], 40)[0]  # (batches of 27 ms: shorter ones read 3 us more, the clocks have not settled)
+            r5 = per_ctx_rows(sw5, [131072], 40)[0]
             f5 = stream_floor(sw5, [131072], FLOOR_CONFIGS[:4])[0]
             result["cfg5"] = dict(r5, workload="64 Q / 8 KV heads, ctx 131072, head-major, graph replays over %d KV slices" % SLICES,
                                   stream_floor_us=f5["us"], floor_ratio=round(f5["us"] / r5["us_per_layer"], 3))
             del sw5
             torch.cuda.empty_cache()
-            # The same workload as the driver-style run of a process of its own (`bench.py --heads 64 --ctx 131072`), whose
-            # arena is the first thing that process allocates: at this length the figure depends on where the two caches lie
-            # (the splits' runs are exactly 1 MiB long and resonate with the memory channels), so both are reported.
-            own = own_process_line(["--heads", "64", "--ctx", "131072", "--no-extras", "--no-cpu-baseline", "--steps", "64", "--warmup", "8"])
-            if own is not None:
-                result["cfg5"]["own_process"] = {"us_per_layer": own["roofline"]["avg_launch_us"], "frac_peak": own["roofline"]["frac"],
-                                                 "command": "python bench.py --heads 64 --ctx 131072 --no-extras --no-cpu-baseline --steps 64 --warmup 8",
-                                                 "note": "the same kernel and workload with the arena allocated first in a fresh process; "
-                                                         "us_per_layer above is this process's arena, allocated after three others were freed"}
             # BASELINE config 4: 36 layers at ctx 4096 + 1 new token, fused QK-Norm + RoPE + append, one HIP graph per token
             ns = argparse.Namespace(stack=36, heads=32, layout=1, stack_mode=5, stack_follow_pos=False, steps=200, warmup=20)
             r4 = stack_result(ns, 4096)
