@@ -123,17 +123,19 @@ int spread_merge_min_splits(int group_pad) {
 // Position-major, runs up to 1 MiB, mask 3. 32 Q / 8 KV heads, with : without: 9.44 : 10.54 us at 8192 positions
 // (512 KiB apart), level at 16384 (1 MiB); everywhere else the wrap-round only costs: 8.32 : 7.99 at 6144, 26.1 : 25.2
 // at 32768, 47.6 : 45.5 at 65536, level at 2048, 4096, 7168, 9216 ... 24576.
-// Head-major, runs from 1 MiB (up to 8 tiles above a multiple of 512 KiB count too: the position moves on by one per
-// token), mask 31. With : without, two layouts of the caches in memory each: 64 Q heads at 131072 positions 81.6 : 88.2
-// and 82.3 : 87.4 us, 32 Q heads 80.4 : 86.3 and 82.5 : 87.4; at 196608 123.3 : 126.8 and 125.7 : 130.2. Not at 65536
-// (512 KiB: 43.3 : 46.1 in one layout, 46.9 : 44.2 in the other), not between the multiples (163840: 108.8 : 100.7),
-// and no gain below (16384: 14.2 : 13.9). LLMI_HIP_STAGGER_MASK overrides the head-major mask (0 = never).
+// Head-major, runs of 512 KiB up to (not including) 2 MiB at a multiple of 512 KiB (up to 8 tiles above one count too:
+// the position moves on by one per token), mask 31. With : without, two seconds of continuous replays each, 64 Q / 8 KV
+// heads: 131072 positions (runs of 1 MiB) 80.0 : 86.3 us in the arena a fresh process allocates and 79.0 : 80.2 in
+// another one, 32 Q heads 79.2 : 85.3 and 78.9 : 79.3; 196608 (1.5 MiB) 118.2 : 121.8; 65536 (512 KiB) 42.15 : 42.6 and
+// 41.75 : 42.0. Not between the multiples (163840: 105.6 : 99.7; 98304: 63.8 : 63.35; 81920: 52.9 : 52.2), not from
+// 2 MiB on (262144: 158.7 : 156.9), not below (32768: 23.27 : 22.63; 40960: 28.5 : 28.2). LLMI_HIP_STAGGER_MASK overrides
+// the head-major mask (0 = never).
 int stagger_mask(int kv_layout, int64_t run_bytes, bool ragged) {
     if (kv_layout == LLMI_KV_LAYOUT_POS_MAJOR)
         return !ragged && run_bytes > 0 && run_bytes % (512 << 10) == 0 && run_bytes <= (1 << 20) ? 3 : 0;
     static const int v = env_int("LLMI_HIP_STAGGER_MASK", 0, 255, -1);
     if (v >= 0) return v;
-    return run_bytes >= (1 << 20) && run_bytes % (512 << 10) < 8 * 4096 ? 31 : 0;
+    return run_bytes >= (512 << 10) && run_bytes < (2 << 20) && run_bytes % (512 << 10) < 8 * 4096 ? 31 : 0;
 }
 
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }

@@ -316,7 +316,7 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     // s & a.stagger tiles into its wave's sequence and wraps round), so that workgroups running in
     // step do not all sit at the same offset of their runs. Where the runs start a multiple of 512 KiB
     // apart, walking them in step keeps hitting the same few memory channels: position-major, 8192
-    // positions, 1.7 us of 13.6; head-major, 131072 positions (runs of 1 MiB), 6 us of 87. Elsewhere it
+    // positions, 1.7 us of 13.6; head-major, 131072 positions (runs of 1 MiB), up to 6 us of 86. Elsewhere it
     // gains nothing or loses, and the bookkeeping costs 0.08 us per call, so the host asks for it by
     // length and it is compiled in only where it is used.
     const int rot = STAGGER ? min(split & a.stagger, max(n_my - 1, 0)) : 0;

@@ -385,7 +385,7 @@ def test_environment_overrides_of_the_dispatch():
 
 def test_stagger_rule_of_the_split_path():
     """Which lengths get the staggered walk: position-major where the splits' runs are exactly 512 KiB or 1 MiB,
-    head-major from 1 MiB at (or a few tiles above) a multiple of 512 KiB; LLMI_HIP_STAGGER_MASK overrides the
+    head-major from 512 KiB to below 2 MiB at (or a few tiles above) a multiple of 512 KiB; LLMI_HIP_STAGGER_MASK overrides the
     head-major mask only (read once per process: a child process per setting)."""
     m = B.lib().llmi_hip_stagger_mask
     K = 1 << 10
@@ -393,11 +393,13 @@ def test_stagger_rule_of_the_split_path():
     assert m(B.KV_LAYOUT_POS_MAJOR, 512 * K, 0) == 3 and m(B.KV_LAYOUT_POS_MAJOR, 1024 * K, 0) == 3
     assert m(B.KV_LAYOUT_POS_MAJOR, 512 * K, 1) == 0 and m(B.KV_LAYOUT_POS_MAJOR, 2048 * K, 0) == 0
     assert m(B.KV_LAYOUT_POS_MAJOR, 384 * K, 0) == 0 and m(B.KV_LAYOUT_POS_MAJOR, 0, 0) == 0
-    # head-major: 131072 positions in 32 splits = 1 MiB runs; 196608 = 1.5 MiB; 65536 = 512 KiB; 163840 = 1.25 MiB
-    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K, 0) == 31 and m(B.KV_LAYOUT_HEAD_MAJOR, 1536 * K, 0) == 31
+    # head-major: 65536 positions in 32 splits = 512 KiB runs; 131072 = 1 MiB; 196608 = 1.5 MiB; 163840 = 1.25 MiB; 262144 = 2 MiB
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 512 * K, 0) == 31 and m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K, 0) == 31
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1536 * K, 0) == 31
     assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K + 7 * 4096, 1) == 31  # the position has moved on by some tokens
     assert m(B.KV_LAYOUT_HEAD_MAJOR, 1024 * K + 8 * 4096, 1) == 0
-    assert m(B.KV_LAYOUT_HEAD_MAJOR, 512 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 1280 * K, 0) == 0
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 1280 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 768 * K, 0) == 0
+    assert m(B.KV_LAYOUT_HEAD_MAJOR, 2048 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 4096 * K, 0) == 0
     assert m(B.KV_LAYOUT_HEAD_MAJOR, 256 * K, 0) == 0 and m(B.KV_LAYOUT_HEAD_MAJOR, 0, 0) == 0
     code = ("import sys; sys.path.insert(0, %r)\n"
             "from llminfer_amd import _binding as B\n"
