@@ -732,6 +732,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="headline sweep only: skip the stream floor, the position-major layout, BASELINE configs 4 and 5 "
                          "and the dispatch check that the default run appends to its JSON line")
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="like --no-extras, and no per-length replays either: every launch of the process is part of the sweep")
     ap.add_argument("--dispatch-check", action="store_true",
                     help="time the automatic plan against forced single-pass / split plans at every --ctx")
     ap.add_argument("--stream-floor", action="store_true",
@@ -856,7 +858,8 @@ def main():
     batch_ms.sort()
     median_ms = batch_ms[len(batch_ms) // 2]
 
-    per_ctx = per_ctx_rows(sw, ctx_list, 40)
+    # (--sweep-only: nothing but the sweep is launched, every length equally often -- what the HBM counters are taken on)
+    per_ctx = [] if args.sweep_only else per_ctx_rows(sw, ctx_list, 40)
     avg_launch_us = ms_per_step * 1e3 / launches_per_step
     avg_launch_bytes = step_bytes / launches_per_step
     achieved = avg_launch_bytes / (avg_launch_us * 1e-6) / 1e9
@@ -889,7 +892,7 @@ def main():
                      "avg_launch_us": round(avg_launch_us, 3), "avg_launch_bytes": int(avg_launch_bytes)},
     }
 
-    if not args.no_extras:
+    if not args.no_extras and not args.sweep_only:
         # What one launch can reach on this machine with the same bytes: the stream-only floor per context.
         floor = stream_floor(sw, ctx_list)
         for row, f in zip(per_ctx, floor):
