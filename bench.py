@@ -330,6 +330,7 @@ def run_stack(args, ctx):
     return 0
 
 
+SWEEP_GRAPH_STEPS = 40
 SETTLE_MS = 40.0
 SETTLE_FIRST_MS = 600.0
 MIN_GRAPH_STEPS = 64
@@ -816,15 +817,17 @@ def main():
         return 0
 
     # ---- the timed region: EXACTLY --steps steps of the whole sweep, after --warmup untimed ones ----------
-    # A graph holds SLICES steps (one per KV slice); a second, shorter graph holds the remainder.
+    # A graph holds SWEEP_GRAPH_STEPS steps (the KV slices in turn, five times round: 240 launches, about what a decode
+    # step of a 36-layer model puts into its graph; between two replays of a graph the device idles for some
+    # microseconds, which short graphs would charge to the kernel); a second, shorter graph holds the remainder.
     def sweep_enqueue(first, n):
         sw.enqueue(ctx_list, first, n)
 
-    g_full = sw.capture(sweep_enqueue, SLICES)
+    g_full = sw.capture(sweep_enqueue, SWEEP_GRAPH_STEPS)
     rem_graphs = {}
 
     def replays_for(k):
-        full, rem = divmod(k, SLICES)
+        full, rem = divmod(k, SWEEP_GRAPH_STEPS)
         seq = [(g_full, full)] if full else []
         if rem:
             if rem not in rem_graphs:
@@ -839,7 +842,7 @@ def main():
     # too. These replays are neither warm-up steps nor timed.
     t_settle = time.perf_counter()
     while time.perf_counter() - t_settle < 0.2:
-        sw.time_replays([(g_full, 20)])
+        sw.time_replays([(g_full, 4)])
     if warm_seq:
         sw.time_replays(warm_seq)
     ms = sw.time_replays(timed_seq)
@@ -854,7 +857,7 @@ def main():
     batch_ms = []
     t_long = time.perf_counter()
     while len(batch_ms) < 5 or (time.perf_counter() - t_long < 0.5 and len(batch_ms) < 400):
-        batch_ms.append(sw.time_replays([(g_full, 10)]) / (10 * SLICES))
+        batch_ms.append(sw.time_replays([(g_full, 2)]) / (2 * SWEEP_GRAPH_STEPS))
     batch_ms.sort()
     median_ms = batch_ms[len(batch_ms) // 2]
 
@@ -877,7 +880,7 @@ def main():
                    "ctx": ctx_list, "bytes_per_step": step_bytes, "kv_layout": args.layout,
                    "workspace_side": "0x%x" % (sw.side & 0xffffffff)},
         "timed_region_s": round(ms * 1e-3, 6),
-        "long_run": {"seconds": round(sum(batch_ms) * 10 * SLICES * 1e-3, 3), "batches": len(batch_ms), "steps_per_batch": 10 * SLICES,
+        "long_run": {"seconds": round(sum(batch_ms) * 2 * SWEEP_GRAPH_STEPS * 1e-3, 3), "batches": len(batch_ms), "steps_per_batch": 2 * SWEEP_GRAPH_STEPS,
                      "ms_per_step_median": round(median_ms, 6), "value_median": round(step_bytes / (median_ms * 1e-3) / 1e9, 1),
                      "ms_per_step_p10": round(batch_ms[len(batch_ms) // 10], 6), "ms_per_step_p90": round(batch_ms[len(batch_ms) * 9 // 10], 6)},
         "us_per_layer_mean": round(avg_launch_us, 3),
