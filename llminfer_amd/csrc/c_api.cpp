@@ -130,12 +130,26 @@ int spread_merge_min_splits(int group_pad) {
 // 41.75 : 42.0. Not between the multiples (163840: 105.6 : 99.7; 98304: 63.8 : 63.35; 81920: 52.9 : 52.2), not from
 // 2 MiB on (262144: 158.7 : 156.9), not below (32768: 23.27 : 22.63; 40960: 28.5 : 28.2). LLMI_HIP_STAGGER_MASK overrides
 // the head-major mask (0 = never).
+static int stagger_mask_override() {
+    static const int v = env_int("LLMI_HIP_STAGGER_MASK", 0, 255, -1);
+    return v;
+}
+
 int stagger_mask(int kv_layout, int64_t run_bytes, bool ragged) {
     if (kv_layout == LLMI_KV_LAYOUT_POS_MAJOR)
         return !ragged && run_bytes > 0 && run_bytes % (512 << 10) == 0 && run_bytes <= (1 << 20) ? 3 : 0;
-    static const int v = env_int("LLMI_HIP_STAGGER_MASK", 0, 255, -1);
+    const int v = stagger_mask_override();
     if (v >= 0) return v;
-    return run_bytes >= (512 << 10) && run_bytes < (2 << 20) && run_bytes % (512 << 10) < 8 * 4096 ? 31 : 0;
+    return head_major_stagger_rule(run_bytes);
+}
+
+// Position read on the device, head-major: the walk's kernels whenever the longest possible run reaches the rule's
+// range (kStaggerByDevice: the kernel decides by the length it finds), the environment's mask as it is, else 0.
+int dyn_stagger(int kv_layout, int64_t max_run_bytes) {
+    if (kv_layout == LLMI_KV_LAYOUT_POS_MAJOR) return 0;
+    const int v = stagger_mask_override();
+    if (v >= 0) return v;
+    return max_run_bytes >= (512 << 10) ? kStaggerByDevice : 0;
 }
 
 int check_launch() { return record_hip_error(hipGetLastError(), "kernel launch"); }

@@ -70,6 +70,20 @@ int spread_merge_min_splits(int group_pad);
 // The mask of the staggered walk (KernelArgs::stagger) for splits whose runs are `run_bytes` long (the shorter ones,
 // when they differ by a tile: `ragged`).
 int stagger_mask(int kv_layout, int64_t run_bytes, bool ragged);
+// ... its head-major rule, for the host and for the kernels that read the position on the device: runs of 512 KiB to
+// below 2 MiB at a multiple of 512 KiB, or up to 8 tiles of 4 KiB above one (the measurements are with stagger_mask).
+#if defined(__HIPCC__)
+#define LLMI_HOST_DEVICE __host__ __device__
+#else
+#define LLMI_HOST_DEVICE
+#endif
+LLMI_HOST_DEVICE constexpr int head_major_stagger_rule(long long run_bytes) {
+    return run_bytes >= (512 << 10) && run_bytes < (2 << 20) && run_bytes % (512 << 10) < 8 * 4096 ? 31 : 0;
+}
+// KernelArgs::stagger of a launch whose position is read on the device: the kernel applies the rule to the length it finds.
+constexpr int kStaggerByDevice = -1;
+// ... and whether such a launch can reach a length the rule applies to at all (else the kernels without the walk run).
+int dyn_stagger(int kv_layout, int64_t max_run_bytes);
 // Polls (each followed by a short sleep) the fused combine waits for the other splits.
 int poll_limit();
 // Testing aid (llmi_hip_set_test_far_home): 1 = every split but the merging one, 2 = every second split stores into

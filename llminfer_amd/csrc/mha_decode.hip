@@ -194,7 +194,9 @@ static int fill_kernel_args(const llmi_mha_args& args, const llmi_mha_plan& plan
         ka.tiles_run = tiles / plan.num_splits;
         ka.tiles_longer = tiles % plan.num_splits;
         // (where the splits' runs start a multiple of 512 KiB apart the splits start their walks at different tiles)
-        ka.stagger = stagger_mask(args.kv_layout, (int64_t)ka.tiles_run * kTile * ka.row_stride * 2, ka.tiles_longer != 0);
+        const int64_t run_bytes = (int64_t)ka.tiles_run * kTile * ka.row_stride * 2;
+        ka.stagger = args.pos_device ? dyn_stagger(args.kv_layout, run_bytes)  // (pos is the upper bound here)
+                                     : stagger_mask(args.kv_layout, run_bytes, ka.tiles_longer != 0);
     }
     ka.scale_log2e = 1.4426950408889634f / sqrtf((float)args.head_dim);
     if (append) {

@@ -319,7 +319,11 @@ __device__ __forceinline__ void mha_decode_body(const KernelArgs& a, OprojState&
     // positions, 1.7 us of 13.6; head-major, 131072 positions (runs of 1 MiB), up to 6 us of 86. Elsewhere it
     // gains nothing or loses, and the bookkeeping costs 0.08 us per call, so the host asks for it by
     // length and it is compiled in only where it is used.
-    const int rot = STAGGER ? min(split & a.stagger, max(n_my - 1, 0)) : 0;
+    // (position read on the device: the host could only say that the rule may apply; what the length found asks for)
+    int rot_mask = a.stagger;
+    if constexpr (DYN && STAGGER)
+        if (rot_mask == kStaggerByDevice) rot_mask = head_major_stagger_rule((long long)run * kTile * a.row_stride * 2);
+    const int rot = STAGGER ? min(split & rot_mask, max(n_my - 1, 0)) : 0;
     auto tile_of = [&](int i) {
         if constexpr (!STAGGER) return wave + i * NW;
         int ii = i + rot;
@@ -1067,12 +1071,16 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
     if constexpr (kHasBySide<G, NW>) {
         if (ka.by_side) {
             if (append) {
-                if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+                if (dyn && ka.stagger)
+                    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
                 else if (ka.stagger)
                     hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, true, true>), grid, dim3(NW * 64), 0, stream, ka);
                 else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
             } else {
-                if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+                if (dyn && ka.stagger)
+                    hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+                else if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
                 else if (ka.stagger)
                     hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, true, true>), grid, dim3(NW * 64), 0, stream, ka);
                 else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
@@ -1081,12 +1089,16 @@ void launch_decode(const KernelArgs& ka, int n_kv, bool append, hipStream_t stre
         }
     }
     if (append) {
-        if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+        if (dyn && ka.stagger && ka.num_splits > 1)
+            hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, true>), grid, dim3(NW * 64), 0, stream, ka);
         else if (ka.stagger && ka.num_splits > 1)
             hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, true, false>), grid, dim3(NW * 64), 0, stream, ka);
     } else {
-        if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);
+        if (dyn && ka.stagger && ka.num_splits > 1)
+            hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true, true>), grid, dim3(NW * 64), 0, stream, ka);
+        else if (dyn) hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else if (ka.stagger && ka.num_splits > 1)
             hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false, true>), grid, dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((mha_decode_kernel<G, NW, kStages, false, false>), grid, dim3(NW * 64), 0, stream, ka);

@@ -97,12 +97,15 @@ def test_one_graph_serves_successive_tokens(oracle, dev):
         assert_parity(from_dev_bf16(out), _oracle_at(oracle, c, p), "replay at pos %d" % p)
 
 
-@pytest.mark.parametrize("layout", [B.KV_LAYOUT_POS_MAJOR, B.KV_LAYOUT_HEAD_MAJOR])
-def test_append_graph_decodes_token_after_token(oracle, dev, layout):
+@pytest.mark.parametrize("layout,n_q,start", [(B.KV_LAYOUT_POS_MAJOR, 32, 250), (B.KV_LAYOUT_HEAD_MAJOR, 32, 250),
+                                               (B.KV_LAYOUT_HEAD_MAJOR, 16, 65533)])
+def test_append_graph_decodes_token_after_token(oracle, dev, layout, n_q, start):
     """llmi_hip_mha_decode_append captured once with a device position: every replay normalises and
     rotates with the sin/cos row of its own position, appends K/V at its own slot and attends over the
-    rows appended so far. The oracle replays the same chain on the host."""
-    n_q, n_kv, d, start, tokens = 32, 8, 128, 250, 6
+    rows appended so far. The oracle replays the same chain on the host. (The long case walks over 65536 cached
+    positions, where the splits' runs are 512 KiB long: the kernel, which only learns the length on the device,
+    staggers its walk from there on and not before.)"""
+    n_kv, d, tokens = 8, 128, 6
     msl = start + tokens + 2
     kv_dim = n_kv * d
     case = synth.make_case(31, n_q=n_q, n_kv=n_kv, ctx=start, max_seq_len=msl)
@@ -166,6 +169,32 @@ def test_append_graph_decodes_token_after_token(oracle, dev, layout):
     want = synth.bf16_bits_to_f32(k_host[0, start:last + 1]).astype(np.float64)
     assert np.all(np.abs(got - want) <= np.abs(want) / 128 + 1e-6)
     assert np.all(kc[0, last + 1:] == 0x7FC0)  # nothing beyond the last appended row was written
+
+
+def test_device_position_at_lengths_with_and_without_the_staggered_walk(oracle, dev):
+    """Head-major, planned for 70001 positions (the longest run exceeds 512 KiB, so the launch uses the kernels that can
+    stagger their walk); the device position then visits lengths where the rule applies (65536 exactly, a few tiles
+    above) and where it does not (below, in between): every result is the oracle's."""
+    n_q, n_kv, max_pos = 16, 8, 70000
+    case = synth.make_case(77, n_q=n_q, n_kv=n_kv, ctx=max_pos + 1, max_seq_len=max_pos + 1)
+    q_d = to_dev(case["q"], dev)
+    k_d = to_dev(synth.to_head_major(case["k"], n_kv), dev)
+    v_d = to_dev(synth.to_head_major(case["v"], n_kv), dev)
+    out = torch.zeros(n_q * 128, dtype=torch.int16, device=dev)
+    out32 = torch.zeros(n_q * 128, dtype=torch.float32, device=dev)
+    ws = torch.full((ops.workspace_bytes(n_q, 128, case["max_seq_len"]) // 4,), float("nan"), dtype=torch.float32, device=dev)
+    pos_t = torch.zeros(1, dtype=torch.int32, device=dev)
+    scal = dict(layer_id=0, pos=max_pos, kv_dim=case["kv_dim"], kv_mul=case["kv_mul"], head_num=n_q, head_dim=128,
+                max_seq_len=case["max_seq_len"], kv_layout=B.KV_LAYOUT_HEAD_MAJOR)
+    for side in (0, ops.workspace_side(ws) or 0x55555555):
+        for p in (65535, 65535 + 37, 65535 + 16 * 8 * 32, 50000, 3000, max_pos):  # (+4096: eight tiles per run above the multiple)
+            pos_t.fill_(p)
+            out.zero_()
+            ops.mha_decode(q_d, k_d, v_d, out, ws, output_f32=out32, pos_device=pos_t, workspace_side=side, **scal)
+            torch.cuda.synchronize()
+            ref = _oracle_at(oracle, case, p)
+            assert_parity(from_dev_bf16(out), ref, "device pos %d, side %x" % (p, side))
+            assert_tap_parity(out32.cpu().numpy(), ref, "device pos %d, side %x" % (p, side))
 
 
 def test_plan_rejects_device_position_with_separate_combine(dev):
