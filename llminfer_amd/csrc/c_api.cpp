@@ -402,6 +402,15 @@ static int compute_units() {
 }
 
 // Validates the arguments and decides between the one-launch form (*fused = true, plan filled) and the pair.
+// Whether the append variant's launch for (m, plan) walks its tiles in step (no staggered walk): the kernels that never
+// stagger (one-launch projection, resident multi-layer launch) only take such lengths, so that they give the bits of the
+// launches they stand for.
+static bool append_walks_in_step(const llmi_mha_args& m, const llmi_mha_plan& plan) {
+    const int tiles = (m.pos + kTile - 1) / kTile;  // (the new token's row does not come from the cache)
+    const int64_t row_bytes = m.kv_layout == LLMI_KV_LAYOUT_POS_MAJOR ? (int64_t)m.kv_dim * 2 : (int64_t)m.head_dim * 2;
+    return stagger_mask(m.kv_layout, (int64_t)(tiles / plan.num_splits) * kTile * row_bytes, tiles % plan.num_splits != 0) == 0;
+}
+
 static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, bool* fused) {
     if (!args) return LLMI_ERR_NULL_POINTER;
     const llmi_mha_append_args& ap = args->attn;
@@ -431,6 +440,7 @@ static int plan_oproj(const llmi_attn_oproj_args* args, llmi_mha_plan* plan, boo
         const int64_t worker_waves = (int64_t)n_kv * (p.num_splits - 1) * p.waves_per_group;
         if (args->hidden > rows_per_wave * worker_waves) return false;
         if ((int64_t)n_kv * p.num_splits > cus) return false;
+        if (!append_walks_in_step(m, p)) return false;
         return m.workspace_bytes >= p.workspace_needed + (size_t)m.head_num * sizeof(uint32_t);
     };
     if (fits(*plan)) {
@@ -498,6 +508,9 @@ static int plan_stack(const llmi_mha_stack_args* args, llmi_mha_plan* plan, bool
     // every workgroup must be resident at once: workgroups wait for each other
     const int cus = compute_units();
     if (cus <= 0 || (int64_t)(m.kv_dim / m.head_dim) * plan->num_splits > cus) return LLMI_OK;
+    // Lengths at which the per-layer launches stagger their walk stay with them: the resident kernel walks in step, so
+    // it would neither be as fast there nor give the same bits (the order of a split's tiles is the order of its sums).
+    if (!append_walks_in_step(m, *plan)) return LLMI_OK;
     *one_launch = true;
     return LLMI_OK;
 }

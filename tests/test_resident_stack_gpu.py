@@ -208,8 +208,11 @@ def test_resident_stack_gives_up_with_nan_instead_of_hanging(dev):
 
 def test_resident_stack_falls_back_to_one_launch_per_layer(dev):
     """Shapes the resident kernel is not built for run as one launch per layer, with the same results: a single pass
-    (short context), groups of eight query heads, more splits than compute units, a workspace without room for the tags."""
-    for n_q, ctx, over in ((32, 100, {}), (64, 2000, {}), (32, 4096, {"num_splits": 64, "force_path": B.PATH_SPLIT_FUSED})):
+    (short context), groups of eight query heads, more splits than compute units, a length at which the per-layer launches
+    stagger their walk (65536 cached positions: the resident kernel walks in step and would not give their bits), a
+    workspace without room for the tags."""
+    for n_q, ctx, over in ((32, 100, {}), (64, 2000, {}), (32, 4096, {"num_splits": 64, "force_path": B.PATH_SPLIT_FUSED}),
+                           (16, 65536, {})):
         st = Stack(dev, 3, ctx, n_q=n_q)
         a, b = st.fresh(), st.fresh()
         st.run_per_layer(a, **over)
